@@ -35,7 +35,7 @@ class KVCacheSpec:
     # k-cache's first v_head_dim dims — only k bytes are allocated
     v_shared: bool = False
     # heterogeneous stacks: (kv_heads, k_dim, v_dim) per cache-owning
-    # layer; when set, num_layers/num_kv_heads/head_dim/v_head_dim above
+    # layer (v_dim 0: keys and values are one cached row); when set, num_layers/num_kv_heads/head_dim/v_head_dim above
     # describe layer 0 only and every layer's cache has its own shape
     layer_shapes: Optional[List[Tuple[int, int, int]]] = None
 

@@ -45,6 +45,10 @@ class SSMLayerSpec:
     # recurrent state [H, Dk, Dv] ("kv": the delta-rule kernels that keep
     # a value-column block per wavefront) or [H, Dv, Dk] ("vk")
     layout: str = "kv"
+    # a recurrence with another state geometry names the per-slot shape
+    # itself (an element-wise gated recurrence: (channels,)); conv_dim 0
+    # = the layer has no short convolution and holds no conv state
+    state_shape: Optional[tuple] = None
 
 
 class SSMPool:
@@ -60,6 +64,8 @@ class SSMPool:
                 num_slots, ls.conv_dim, max(ls.conv_kernel - 1, 1),
                 dtype=dtype, device=device) for ls in spec.layers]
             self.ssm_state = [torch.zeros(
+                (num_slots,) + tuple(ls.state_shape)
+                if ls.state_shape is not None else
                 (num_slots, ls.num_v_heads) + (
                     (ls.head_k_dim, ls.head_v_dim) if ls.layout == "kv"
                     else (ls.head_v_dim, ls.head_k_dim)),

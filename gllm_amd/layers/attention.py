@@ -60,7 +60,14 @@ class WindowAttention(nn.Module):
       in the paged cache
     * position i sees j <= i with i - j < ``window`` or j < ``keep_first``
       (window 0 = plain causal)
-    * ``sink``: softmax denominator 1 + sum exp(s)
+    * ``sink``: softmax denominator 1 + sum exp(s); ``sink="learned"``:
+      exp(sinks[h]) + sum exp(s) with the fp32 parameter ``sinks`` [H]
+    * ``qk_norm`` False: q and k are rotated only (no per-head norm)
+    * ``softcap`` > 0: scores become cap * tanh(score / cap)
+    * ``value_rotary`` (a PairRotary over all of ``v_head_dim``): the
+      value of position j enters the cache turned by j, and each head's
+      weighted sum at position i is turned back by i, so what a query
+      receives from a key depends on their distance only
     * ``kv_source``: cache index of ANOTHER layer whose keys and values
       this layer attends over; such a layer owns no k/v tensors and
       stores nothing (``owns_kv`` False)
@@ -70,9 +77,11 @@ class WindowAttention(nn.Module):
 
     def __init__(self, layer_idx: int, num_heads: int, num_kv_heads: int,
                  head_dim: int, v_head_dim: int, scale: float, eps: float,
-                 window: int = 0, keep_first: int = 0, sink: bool = False,
+                 window: int = 0, keep_first: int = 0, sink=False,
                  rotary: Optional[nn.Module] = None, owns_kv: bool = True,
-                 params_dtype=None):
+                 params_dtype=None, qk_norm: bool = True,
+                 softcap: float = 0.0,
+                 value_rotary: Optional[nn.Module] = None):
         super().__init__()
         dtype = params_dtype or torch.get_default_dtype()
         self.layer_idx = layer_idx       # cache this layer reads
@@ -84,14 +93,28 @@ class WindowAttention(nn.Module):
         self.eps = eps
         self.window = window
         self.keep_first = keep_first
-        self.sink = sink
+        self.sink = bool(sink) and sink != "learned"
         self.rotary = rotary
         self.owns_kv = owns_kv
-        self.q_norm = nn.Parameter(torch.ones(head_dim, dtype=dtype),
-                                   requires_grad=False)
-        if owns_kv:
-            self.k_norm = nn.Parameter(torch.ones(head_dim, dtype=dtype),
+        self.qk_norm = qk_norm
+        self.softcap = float(softcap or 0.0)
+        self.value_rotary = value_rotary
+        if value_rotary is not None:
+            assert value_rotary.rot_dims == v_head_dim
+        if qk_norm:
+            self.q_norm = nn.Parameter(torch.ones(head_dim, dtype=dtype),
                                        requires_grad=False)
+            if owns_kv:
+                self.k_norm = nn.Parameter(
+                    torch.ones(head_dim, dtype=dtype), requires_grad=False)
+        else:
+            self.q_norm = self.k_norm = None
+        if sink == "learned":
+            self.sinks = nn.Parameter(
+                torch.zeros(num_heads, dtype=torch.float32),
+                requires_grad=False)
+        else:
+            self.sinks = None
         self._no_rot = None
 
     def _freqs(self, device):
@@ -103,31 +126,50 @@ class WindowAttention(nn.Module):
 
     def forward(self, q: torch.Tensor, k: Optional[torch.Tensor],
                 v: Optional[torch.Tensor], gate: Optional[torch.Tensor],
-                fctx: ForwardContext) -> torch.Tensor:
+                fctx: ForwardContext, out: Optional[torch.Tensor] = None,
+                out_scale: float = 1.0) -> torch.Tensor:
         """q [T, H*D], k [T, G*D], v [T, G*Dv], gate [T, H*Dv] (row
-        views of a merged projection are fine). Returns [T, H*Dv]."""
+        views of a merged projection are fine). Returns [T, H*Dv],
+        multiplied by ``out_scale`` and written into ``out`` (which may
+        be a column block of a wider buffer) when those are given."""
         T = q.shape[0]
         if fctx.is_profile_run:
+            if out is not None:
+                out.zero_()
+                return out
             return q.new_zeros(T, self.num_heads * self.v_head_dim)
         k_cache = fctx.k_caches[self.layer_idx]
         v_cache = fctx.v_caches[self.layer_idx]
         freqs, mag, rot_dims = self._freqs(q.device)
+        vrot = self.value_rotary
+        vfreqs = vrot.freqs if vrot is not None else None
         if self.owns_kv:
             ops.qk_norm_rope_store(
                 q, k, v, self.q_norm, self.k_norm, fctx.positions,
                 fctx.slot_mapping, freqs, mag, rot_dims, k_cache, v_cache,
                 self.num_heads, self.num_kv_heads, self.head_dim,
-                self.v_head_dim, self.eps)
+                self.v_head_dim, self.eps, do_norm=self.qk_norm,
+                v_freqs=vfreqs)
         else:
             ops.qk_norm_rope_store(
                 q, None, None, self.q_norm, None, fctx.positions,
                 fctx.slot_mapping, freqs, mag, rot_dims, None, None,
                 self.num_heads, self.num_kv_heads, self.head_dim,
-                self.v_head_dim, self.eps)
-        return ops.window_attention(
+                self.v_head_dim, self.eps, do_norm=self.qk_norm)
+        o = ops.window_attention(
             q, gate, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
             fctx.query_start_loc, self.scale, self.window,
-            self.keep_first, self.sink, fctx.max_query_len)
+            self.keep_first, self.sink, fctx.max_query_len,
+            sinks=self.sinks, softcap=self.softcap)
+        if vrot is not None:
+            # turn every head's sum back by the query's own position
+            return ops.rotate_scale_rows(
+                o, fctx.positions, vfreqs, self.num_heads, self.v_head_dim,
+                -1.0, out_scale, out=out)
+        if out is not None:
+            out.copy_(o if out_scale == 1.0 else o * out_scale)
+            return out
+        return o if out_scale == 1.0 else o * out_scale
 
 
 class TalkingHeadsAttention(nn.Module):
@@ -199,3 +241,77 @@ class TalkingHeadsAttention(nn.Module):
             q, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
             fctx.query_start_loc, self.scale, self.talk, self.sink,
             fctx.max_query_len)
+
+
+class LatentAttention(nn.Module):
+    """Causal attention whose keys and values are up-projections of one
+    cached low-rank latent per token, without positions.
+
+        c_t   = RMSnorm(W_dkv h_t)                  (the only cached row)
+        k_j,h = W_uk,h c_j      v_j,h = W_uv,h c_j
+        s     = scale * q_i,h . k_j,h,  softmax over j <= i
+
+    The up-projections are never applied to the cache: the query is
+    carried into the latent space (q~ = W_uk,h^T q, so q~ . c = q . k),
+    attention runs over the latent rows themselves as one shared
+    key/value head, and the per-head weighted latent is brought to the
+    value space afterwards (W_uv,h applied to the sum). The cache of the
+    layer is ``[pages, page, 1, rank]`` and serves as key and value
+    cache at once.
+
+    ``owns_kv`` False: the layer has no W_dkv and attends over the
+    latent another layer cached (``layer_idx`` names that cache), with
+    up-projections of its own.
+
+    ``w_uk`` [H, D, rank] and ``w_uv`` [H, Dv, rank] are parameters of
+    this module; the down projections and their norms live in the
+    caller's merged projection.
+    """
+
+    def __init__(self, layer_idx: int, num_heads: int, head_dim: int,
+                 v_head_dim: int, rank: int, scale: float, eps: float,
+                 owns_kv: bool = True, params_dtype=None):
+        super().__init__()
+        dtype = params_dtype or torch.get_default_dtype()
+        self.layer_idx = layer_idx
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+        self.v_head_dim = v_head_dim
+        self.rank = rank
+        self.scale = scale
+        self.eps = eps
+        self.owns_kv = owns_kv
+        self.w_uk = nn.Parameter(
+            torch.empty(num_heads, head_dim, rank, dtype=dtype),
+            requires_grad=False)
+        self.w_uv = nn.Parameter(
+            torch.empty(num_heads, v_head_dim, rank, dtype=dtype),
+            requires_grad=False)
+        if owns_kv:
+            self.kv_norm = nn.Parameter(torch.ones(rank, dtype=dtype),
+                                        requires_grad=False)
+
+    def forward(self, q: torch.Tensor, ckv: Optional[torch.Tensor],
+                fctx: ForwardContext) -> torch.Tensor:
+        """q [T, H*D]; ckv [T, rank] = W_dkv h before its norm (None for
+        a layer that reads another layer's latent). Returns [T, H*Dv]."""
+        T = q.shape[0]
+        H, D, Dv, R = self.num_heads, self.head_dim, self.v_head_dim, \
+            self.rank
+        if fctx.is_profile_run:
+            return q.new_zeros(T, H * Dv)
+        cache = fctx.k_caches[self.layer_idx]
+        if self.owns_kv:
+            ops.rms_weight_store(ckv, self.kv_norm, self.eps, cache,
+                                 fctx.slot_mapping)
+        # q~[t, h] = W_uk,h^T q[t, h]
+        q_lat = torch.bmm(q.reshape(T, H, D).transpose(0, 1), self.w_uk)
+        q_lat = q_lat.transpose(0, 1).reshape(T, H * R)
+        o_lat = ops.window_attention(
+            q_lat, None, cache, cache, fctx.block_table, fctx.seq_lens,
+            fctx.query_start_loc, self.scale, 0, 0, False,
+            fctx.max_query_len)
+        # o[t, h] = W_uv,h o~[t, h]
+        o = torch.bmm(o_lat.reshape(T, H, R).transpose(0, 1),
+                      self.w_uv.transpose(1, 2))
+        return o.transpose(0, 1).reshape(T, H * Dv)

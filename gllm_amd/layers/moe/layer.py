@@ -24,16 +24,22 @@ class FusedMoE(nn.Module):
                  intermediate_size: int, renormalize: bool = True,
                  use_ep: bool = False, params_dtype=None,
                  activation: str = "silu_glu",
-                 fp32_routing_weights: bool = False):
+                 fp32_routing_weights: bool = False,
+                 act_limit: float = 0.0, act_alpha: float = 1.702):
         """``activation``: "silu_glu" — gated experts, w13 holds gate
         and up rows, act = silu(gate) * up; "relu2" — ungated experts,
-        w13 holds the up rows only, act = max(z, 0)^2.
+        w13 holds the up rows only, act = max(z, 0)^2; "swiglu_clamp" —
+        gated experts with clamped pre-activations: g = min(gate,
+        act_limit), u = clamp(up, +-act_limit), act = g * sigmoid(
+        act_alpha g) * (u + 1).
         ``fp32_routing_weights``: keep the routing weights in fp32 up to
         the weighted sum instead of rounding them to the model dtype."""
         super().__init__()
-        assert activation in ("silu_glu", "relu2")
+        assert activation in ("silu_glu", "relu2", "swiglu_clamp")
         self.activation = activation
-        self.gated = activation == "silu_glu"
+        self.act_args = (float(act_limit), float(act_alpha)) \
+            if activation == "swiglu_clamp" else ()
+        self.gated = activation != "relu2"
         self.fp32_routing_weights = fp32_routing_weights
         dtype = params_dtype or torch.get_default_dtype()
         self.num_experts = num_experts
@@ -178,7 +184,7 @@ class FusedMoE(nn.Module):
                     x.contiguous(), self.w13_weight, self.w2_weight,
                     weights, ids, expert_start=self.expert_start,
                     num_global_experts=self.num_experts,
-                    activation=self.activation)
+                    activation=self.activation, act_args=self.act_args)
             if (self.fp8_block == (128, 128)
                     and x.shape[1] % 128 == 0
                     and self.intermediate_per_rank % 128 == 0):
@@ -230,7 +236,10 @@ class FusedMoE(nn.Module):
             else:
                 w13, w2 = self.w13_weight[lid], self.w2_weight[lid]
             h = ops.linear(xe, w13)
-            h = ops.silu_and_mul(h) if self.gated else ops.relu2(h)
+            if self.activation == "swiglu_clamp":
+                h = ops.clamp_swiglu(h, *self.act_args)
+            else:
+                h = ops.silu_and_mul(h) if self.gated else ops.relu2(h)
             ye = ops.linear(h, w2)
             w = flat_w[sel].unsqueeze(-1)
             if w.dtype != ye.dtype:       # fp32 routing weights

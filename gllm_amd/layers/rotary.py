@@ -208,6 +208,12 @@ class PairRotary(nn.Module):
     (ramp 0) keep their frequency, with a linear ramp between the
     correction dims of ``fast`` and ``slow`` rotations, and cos/sin are
     scaled by 0.1 ln(factor) + 1.
+
+    ``scaling`` = dict(factor, low, high, original) instead selects the
+    wavelength rule: with l = 2 pi / f, pairs with l < original/high
+    keep f, pairs with l > original/low run at f / factor, and between
+    the two f is blended linearly in s = (original/l - low) /
+    (high - low): (1 - s) f / factor + s f. cos/sin keep magnitude 1.
     """
 
     def __init__(self, rot_dims: int, base: float,
@@ -219,7 +225,17 @@ class PairRotary(nn.Module):
         freqs = torch.pow(torch.tensor(float(base), dtype=torch.float64),
                           -2.0 * i / max(rot_dims, 1))
         self.mag = 1.0
-        if scaling:
+        if scaling and "low" in scaling:
+            factor = float(scaling["factor"])
+            low, high = float(scaling["low"]), float(scaling["high"])
+            orig = float(scaling["original"])
+            wl = 2 * math.pi / freqs
+            s = (orig / wl - low) / (high - low)
+            blend = (1.0 - s) * freqs / factor + s * freqs
+            freqs = torch.where(wl < orig / high, freqs,
+                                torch.where(wl > orig / low,
+                                            freqs / factor, blend))
+        elif scaling:
             factor = float(scaling["factor"])
             orig = float(scaling["original"])
 

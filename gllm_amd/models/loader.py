@@ -35,7 +35,9 @@ def get_arch_registry():
                                           Qwen3_5VLForCausalLM)
     from gllm_amd.models.sudevik import SudevikForCausalLM
     from gllm_amd.models.gukirax import GukiraxForCausalLM
+    from gllm_amd.models.gopetar import GopetarForCausalLM
     return {
+        "Gopetar": GopetarForCausalLM,
         "Sudevik": SudevikForCausalLM,
         "Gukirax": GukiraxForCausalLM,
         "Qwen2VLForConditionalGeneration": Qwen2VLForCausalLM,

@@ -208,10 +208,13 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
               topk_weights: torch.Tensor, topk_ids: torch.Tensor,
               expert_start: int = 0,
               num_global_experts: Optional[int] = None,
-              activation: str = "silu_glu") -> torch.Tensor:
+              activation: str = "silu_glu",
+              act_args: tuple = ()) -> torch.Tensor:
     """Grouped-GEMM fused MoE on the gfx950 kernels (GPU, bf16).
-    ``activation``: "silu_glu" (w13 = gate | up rows) or "relu2"
-    (ungated experts, w13 = up rows only, act = max(z, 0)^2).
+    ``activation``: "silu_glu" (w13 = gate | up rows), "relu2"
+    (ungated experts, w13 = up rows only, act = max(z, 0)^2) or
+    "swiglu_clamp" (w13 = gate | up rows, ``act_args`` = (limit,
+    alpha): min(g, limit) * sigmoid(alpha g) * (clamp(u) + 1)).
 
     Reference fused_experts_impl (fused_moe_triton/fused_moe.py:779):
     align -> GEMM1 -> silu_and_mul -> GEMM2 (weighted scatter) -> sum.
@@ -251,7 +254,12 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
     inter1 = torch.empty(rows_pad, two_i, dtype=x.dtype, device=dev)
     k.moe_gemm(inter1, x, w13, sorted_ids, expert_blocks, n_post, None,
                n_pairs, topk, gemm_m, False)
-    act = relu2(inter1) if activation == "relu2" else silu_and_mul(inter1)
+    if activation == "relu2":
+        act = relu2(inter1)
+    elif activation == "swiglu_clamp":
+        act = clamp_swiglu(inter1, *act_args)
+    else:
+        act = silu_and_mul(inter1)
     # zero-filled: pairs routed to non-local experts (EP shards) or to
     # the DP padding id -1 are dropped by the align kernel and must
     # contribute zeros
@@ -773,7 +781,8 @@ def residual_layernorm(x: torch.Tensor, y: torch.Tensor, w_post, b_post,
 # --------------------------------------------------------------- windowed attn
 def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
                        mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
-                       half_layout=False, norm_last=False):
+                       half_layout=False, norm_last=False, do_norm=True,
+                       v_freqs=None):
     """Fused per-head q/k RMS norm, rotary (per-pair frequency table
     ``freqs`` fp64, cos/sin scaled by ``mag``) and paged K/V store.
     q [T, H*D] is updated in place (may be a column slice of a merged
@@ -782,25 +791,115 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
     ``q_w``/``k_w`` None: unit-RMS heads without a weight.
     ``half_layout``: dimension i rotates with i + rot_dims/2 (the
     default pairs 2i with 2i+1). ``norm_last``: rotate, then norm.
-    ``v`` may be ``k`` itself (values = keys as projected)."""
+    ``v`` may be ``k`` itself (values = keys as projected).
+    ``do_norm`` False: rotary and store only. ``v_freqs`` (fp64
+    [Dv/2]): each value row is turned by its own position over all of
+    Dv (same pair layout) on its way into the cache."""
     if q.is_cuda:
         _seq_kernels().qk_norm_rope_store(
             q, k, v, q_w, k_w, positions, slot_mapping, freqs, mag,
             rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
-            bool(half_layout), bool(norm_last))
+            bool(half_layout), bool(norm_last), bool(do_norm), v_freqs)
         return
     torch_ref.qk_norm_rope_store(q, k, v, q_w, k_w, positions,
                                  slot_mapping, freqs, mag, rot_dims,
                                  k_cache, v_cache, H, G, D, Dv, eps,
-                                 half_layout, norm_last)
+                                 half_layout, norm_last, do_norm, v_freqs)
+
+
+def rotate_scale_rows(x, positions, freqs, heads, D, sign=1.0, scale=1.0,
+                      half_layout=False, out=None) -> torch.Tensor:
+    """Turn the pairs of every head row of x [T, heads*D] by
+    sign * position * freqs[m] and scale the result (sign -1 undoes the
+    turn that rotated values carry). ``out`` may be a column block of a
+    wider buffer."""
+    if x.is_cuda:
+        if out is None:
+            out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _seq_kernels().rotate_scale_rows(out, x, positions, freqs, heads, D,
+                                         float(sign), float(scale),
+                                         bool(half_layout))
+        return out
+    return torch_ref.rotate_scale_rows(x, positions, freqs, heads, D, sign,
+                                       scale, half_layout, out)
+
+
+def rms_weight_store(x, w, eps, cache=None, slot_mapping=None):
+    """x / rms(x) * w per row (fp32 inside, x's dtype out); with
+    ``cache`` [pages, page, 1, n] the normed rows are also scattered
+    into their paged slots (a cached low-rank latent)."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _seq_kernels().rms_weight_store(out, x, w, eps, cache, slot_mapping)
+        return out
+    return torch_ref.rms_weight_store(x, w, eps, cache, slot_mapping)
+
+
+# --------------------------------------------------------------- streams
+def hyper_streams(xs, y=None, y2=None, gate=None, mix=None, out_w=None,
+                  read=None, dtype=None):
+    """Hyper-connection residual xs [S, T, W] fp32.
+
+    Write (``y`` given, in place): x_t <- sum_s mix[s, t] x_s +
+    out_w[t] * (y + sigmoid(gate) * y2), all streams from the old ones;
+    y2 / gate ([T, 1] logits) optional. Read (``read`` = (in_w [S],
+    gain [1], eps)): returns gain * u / rms(u) in ``dtype`` with
+    u = sum_s in_w[s] x_s — of the updated streams when both are asked
+    for (one launch per sublayer boundary)."""
+    if xs.is_cuda:
+        h = None
+        in_w = gain = None
+        eps = 0.0
+        if read is not None:
+            in_w, gain, eps = read
+            h = torch.empty(xs.shape[1:], dtype=dtype, device=xs.device)
+        _seq_kernels().hyper_streams(xs, y, y2, gate, mix, out_w, h, in_w,
+                                     gain, eps)
+        return h
+    return torch_ref.hyper_streams(xs, y, y2, gate, mix, out_w, read, dtype)
+
+
+# --------------------------------------------------------------- minGRU
+def mingru_varlen(zx, gp, state, slots, has_init, query_start_loc,
+                  scale=1.0, max_query_len=0, out=None) -> torch.Tensor:
+    """Ragged minGRU (prompt portions and decode tokens in one
+    launch): zx [T, 2C] update-gate | candidate pre-activations, gp
+    [T, C] read-out gate logits, fp32 state [slots, C] in place.
+    Returns scale * S_t * silu(gp_t) in zx's dtype ([T, C]; ``out`` may
+    be a column block of a wider buffer)."""
+    if zx.is_cuda:
+        if out is None:
+            out = torch.empty(gp.shape, dtype=zx.dtype, device=zx.device)
+        _seq_kernels().mingru_varlen(out, zx, gp, state, slots, has_init,
+                                     query_start_loc, float(scale),
+                                     int(max_query_len))
+        return out
+    return torch_ref.mingru_varlen(zx, gp, state, slots, has_init,
+                                   query_start_loc, scale, out)
+
+
+def clamp_swiglu(x: torch.Tensor, limit: float,
+                 alpha: float = 1.702) -> torch.Tensor:
+    """x [rows, 2d] = gate | up -> min(g, limit) * sigmoid(alpha g) *
+    (clamp(u, -limit, limit) + 1)."""
+    if x.is_cuda:
+        out = torch.empty(x.shape[0], x.shape[1] // 2, dtype=x.dtype,
+                          device=x.device)
+        _seq_kernels().clamp_swiglu(out, x, float(limit), float(alpha))
+        return out
+    return torch_ref.clamp_swiglu(x, limit, alpha)
 
 
 def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
                      query_start_loc, scale, window=0, keep_first=0,
-                     sink=False, max_query_len=0) -> torch.Tensor:
+                     sink=False, max_query_len=0, sinks=None,
+                     softcap=0.0) -> torch.Tensor:
     """Ragged paged attention over K [pages, page, G, D] / V [.., Dv]:
     sliding window with kept first tokens, optional softmax sink (+1 in
-    the denominator) and fused sigmoid output gate. Returns [T, H*Dv].
+    the denominator; ``sinks`` fp32 [H]: exp(sinks[h]) instead), tanh
+    score cap (``softcap`` > 0: cap * tanh(s / cap)) and fused sigmoid
+    output gate. K and V may be the same tensor (attention over a
+    cached latent). Returns [T, H*Dv].
 
     Batches that hold prompt portions (``max_query_len`` > 1) in bf16
     with D == Dv in {64, 128} run the MFMA tile kernel shared with
@@ -818,23 +917,24 @@ def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
             _seq_kernels().window_attention_mfma(
                 out, q, gate, k_cache, v_cache, block_table, seq_lens,
                 query_start_loc, max_query_len, scale, window, keep_first,
-                sink)
+                sink, sinks, softcap)
             return out
         if (max_query_len == 1 and q.dtype == torch.bfloat16 and D == Dv
                 and _seq_kernels().window_attention_decode(
                     out, q, gate, k_cache, v_cache, block_table, seq_lens,
-                    scale, window, keep_first, sink)):
+                    scale, window, keep_first, sink, sinks, softcap)):
             # decode-only batch on the split-KV kernels shared with
             # paged_attention (one workgroup per GQA group and KV split)
             return out
         _seq_kernels().window_attention(
             out, q, gate, k_cache, v_cache, block_table, seq_lens,
-            query_start_loc, scale, window, keep_first, sink)
+            query_start_loc, scale, window, keep_first, sink, sinks,
+            softcap)
         return out
     return torch_ref.window_attention(q, gate, k_cache, v_cache,
                                       block_table, seq_lens,
                                       query_start_loc, scale, window,
-                                      keep_first, sink)
+                                      keep_first, sink, sinks, softcap)
 
 
 # --------------------------------------------------------------- talking heads

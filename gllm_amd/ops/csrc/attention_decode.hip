@@ -34,7 +34,8 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_kernel(
     const int *__restrict__ block_table,  // [B, max_pages]
     const int *__restrict__ seq_lens,     // [B]
     int max_pages, int page_size, int num_kv_heads, float scale,
-    int num_splits, long q_stride, int window, int keep_first) {
+    int num_splits, long q_stride, int window, int keep_first,
+    float softcap) {
   const int b = blockIdx.x;
   const int kvh = blockIdx.y;
   const int split = blockIdx.z;
@@ -127,7 +128,11 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_kernel(
 #pragma unroll
       for (int h = 0; h < G; ++h) {
         float v = group_reduce_sum<D / 8>(dot[h]);
-        if (dlane == 0 && tt < c_len) s_scores[h][tt] = v * scale;
+        if (dlane == 0 && tt < c_len) {
+          v *= scale;
+          if (softcap > 0.f) v = softcap * tanhf(v / softcap);
+          s_scores[h][tt] = v;
+        }
       }
     }
     __syncthreads();
@@ -263,7 +268,8 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_mfma_kernel(
     const __hip_bfloat16 *__restrict__ v_cache,
     const int *__restrict__ block_table, const int *__restrict__ seq_lens,
     int max_pages, int page_size, int num_kv_heads, float scale,
-    int num_splits, long q_stride, int window, int keep_first) {
+    int num_splits, long q_stride, int window, int keep_first,
+    float softcap) {
   constexpr int D = 128;
   constexpr int CK = 64;            // kv tokens per chunk
   const int b = blockIdx.x;
@@ -374,6 +380,7 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_mfma_kernel(
       const int tok = wave * 16 + l16;
       if (h < G && tok < CK) {
         float sv = s_frag[r] * scale;
+        if (softcap > 0.f) sv = softcap * tanhf(sv / softcap);
         if (c0 + tok >= t1) sv = -INFINITY;
         s_scores[h][tok] = sv;
       }
@@ -478,15 +485,19 @@ __global__ void decode_merge_kernel(
     const float *__restrict__ partial_out,  // [S, B, Hq, D]
     const float *__restrict__ partial_lse,  // [S, B, Hq]
     int num_splits, int Hq, int sink,
-    const __hip_bfloat16 *__restrict__ gate, long gate_stride) {
+    const __hip_bfloat16 *__restrict__ gate, long gate_stride,
+    const float *__restrict__ sinks) {
   const int b = blockIdx.x, h = blockIdx.y;
   const int d = threadIdx.x;
   const int B = gridDim.x;
-  // sink: one more "partial" with lse 0 and no value
-  float mx = sink ? 0.f : -INFINITY;
+  // sink: one more "partial" with lse 0 (or the head's learned score)
+  // and no value
+  const float sk = sinks ? sinks[h] : 0.f;
+  sink = sink || sinks != nullptr;
+  float mx = sink ? sk : -INFINITY;
   for (int s = 0; s < num_splits; ++s)
     mx = fmaxf(mx, partial_lse[((long)s * B + b) * Hq + h]);
-  float denom = sink ? __expf(-mx) : 0.f, o = 0.f;
+  float denom = sink ? __expf(sk - mx) : 0.f, o = 0.f;
   for (int s = 0; s < num_splits; ++s) {
     const float lse = partial_lse[((long)s * B + b) * Hq + h];
     if (lse == -INFINITY) continue;
@@ -510,7 +521,8 @@ void launch_decode(torch::Tensor &out, const torch::Tensor &q,
                    const torch::Tensor &seq_lens, float scale,
                    int max_seq_len, long q_stride, int window,
                    int keep_first = 0, bool sink = false,
-                   const void *gate = nullptr, long gate_stride = 0) {
+                   const void *gate = nullptr, long gate_stride = 0,
+                   const float *sinks = nullptr, float softcap = 0.f) {
   const int B = q.size(0);
   const int Hkv = k_cache.size(2);
   const int Hq = Hkv * G;
@@ -546,7 +558,7 @@ void launch_decode(torch::Tensor &out, const torch::Tensor &q,
                        block_table.data_ptr<int>(),
                        seq_lens.data_ptr<int>(), (int)block_table.stride(0),
                        (int)k_cache.size(1), Hkv, scale, splits, q_stride,
-                       window, keep_first);
+                       window, keep_first, softcap);
   } else {
     hipLaunchKernelGGL((paged_decode_kernel<D, G, CHUNK>),
                        dim3(B, Hkv, zdim), dim3(BLOCK), 0, stream,
@@ -556,14 +568,14 @@ void launch_decode(torch::Tensor &out, const torch::Tensor &q,
                        (const __hip_bfloat16 *)v_cache.data_ptr(),
                        block_table.data_ptr<int>(), seq_lens.data_ptr<int>(),
                        (int)block_table.stride(0), (int)k_cache.size(1), Hkv,
-                       scale, splits, q_stride, window, keep_first);
+                       scale, splits, q_stride, window, keep_first, softcap);
   }
   HIP_CHECK_KERNEL();
   hipLaunchKernelGGL((decode_merge_kernel<D>), dim3(B, Hq), dim3(D), 0,
                      stream, (__hip_bfloat16 *)out.data_ptr(),
                      partial.data_ptr<float>(), lse.data_ptr<float>(), zdim,
                      Hq, sink ? 1 : 0, (const __hip_bfloat16 *)gate,
-                     gate_stride);
+                     gate_stride, sinks);
   HIP_CHECK_KERNEL();
 }
 
@@ -611,7 +623,9 @@ bool window_attention_decode(torch::Tensor out, torch::Tensor q,
                              torch::Tensor k_cache, torch::Tensor v_cache,
                              torch::Tensor block_table,
                              torch::Tensor seq_lens, double scale,
-                             long window, long keep_first, bool sink) {
+                             long window, long keep_first, bool sink,
+                             c10::optional<torch::Tensor> sinks,
+                             double softcap) {
   const int B = q.size(0);
   if (B == 0) return true;
   const int D = k_cache.size(3);
@@ -638,12 +652,19 @@ bool window_attention_decode(torch::Tensor out, torch::Tensor q,
     gp = gate->data_ptr();
     gs = gate->stride(0);
   }
+  const float *sp = nullptr;
+  if (sinks.has_value()) {
+    TORCH_CHECK(sinks->scalar_type() == at::kFloat && sinks->is_contiguous() &&
+                sinks->numel() == (long)Hkv * G, "sinks: fp32 [H]");
+    sp = sinks->data_ptr<float>();
+  }
   const int max_seq = k_cache.size(0) * k_cache.size(1);
 #define CASE(DD, GG)                                                       \
   if (D == DD && G == GG) {                                                \
     launch_decode<DD, GG>(out, q, k_cache, v_cache, block_table, seq_lens, \
                           (float)scale, max_seq, q.stride(0), (int)window, \
-                          (int)keep_first, sink, gp, gs);                  \
+                          (int)keep_first, sink, gp, gs, sp,               \
+                          (float)softcap);                                 \
     return true;                                                           \
   }
   CASE(128, 1) CASE(128, 2) CASE(128, 4) CASE(128, 5) CASE(128, 8)

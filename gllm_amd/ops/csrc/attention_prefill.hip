@@ -56,7 +56,10 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
     // score-0, value-less key to the softmax (denominator 1 + sum exp);
     // gate multiplies the output by sigmoid(gate[t, h*D + d])
     int keep_first, int sink, const __hip_bfloat16 *__restrict__ gate,
-    long gate_stride) {
+    long gate_stride,
+    // per-head learned sink scores (in place of 0) and a tanh cap
+    // cap * tanh(s / cap) on the scaled scores (0 = none)
+    const float *__restrict__ sinks, float softcap) {
   const int tile = blockIdx.x;
   const int b = blockIdx.y;
   const int h = blockIdx.z;
@@ -103,8 +106,8 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     // the sink enters as an already-seen key of score 0
-    m_run[r] = sink ? 0.f : -INFINITY;
-    l_run[r] = sink ? 1.f : 0.f;
+    m_run[r] = sinks ? sinks[h] : (sink ? 0.f : -INFINITY);
+    l_run[r] = (sink || sinks) ? 1.f : 0.f;
   }
   mfma_f4 o_acc[NT];
 #pragma unroll
@@ -206,6 +209,7 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
 #pragma unroll
         for (int f = 0; f < NF; ++f) {
           sv[f] = s_frag[f][r] * scale;
+          if (softcap > 0.f) sv[f] = softcap * tanhf(sv[f] / softcap);
           mx = fmaxf(mx, sv[f]);
         }
       } else {
@@ -213,6 +217,7 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
         for (int f = 0; f < NF; ++f) {
           const int kvp = kv0 + f * 16 + l16;
           float s = s_frag[f][r] * scale;
+          if (softcap > 0.f) s = softcap * tanhf(s / softcap);
           if (qrow >= q_len || kvp > qpos || kvp >= seq_len)
             s = -INFINITY;
           if (window > 0 && kvp <= qpos - window && kvp >= keep_first)
@@ -315,7 +320,8 @@ void launch_prefill(torch::Tensor &out, torch::Tensor &q, int Hq, int D,
                     torch::Tensor &seq_lens, torch::Tensor &query_start_loc,
                     long max_query_len, double scale, long window,
                     long keep_first, bool sink, const void *gate,
-                    long gate_stride) {
+                    long gate_stride, const float *sinks = nullptr,
+                    float softcap = 0.f) {
   const int Hkv = k_cache.size(2);
   const int B = seq_lens.size(0);
   const int q_tiles = (int)((max_query_len + BQ - 1) / BQ);
@@ -332,7 +338,8 @@ void launch_prefill(torch::Tensor &out, torch::Tensor &q, int Hq, int D,
                      (int)block_table.stride(0), (int)k_cache.size(1), Hq,   \
                      Hkv, (float)scale, q_stride, (int)window,               \
                      (int)keep_first, sink ? 1 : 0,                          \
-                     (const __hip_bfloat16 *)gate, gate_stride)
+                     (const __hip_bfloat16 *)gate, gate_stride, sinks,       \
+                     softcap)
   if (D == 128) RUN(128);
   else if (D == 64) RUN(64);
   else TORCH_CHECK(false, "prefill attn: head_dim ", D, " unsupported");
@@ -368,7 +375,8 @@ void window_attention_mfma(torch::Tensor out, torch::Tensor q,
                            torch::Tensor block_table, torch::Tensor seq_lens,
                            torch::Tensor query_start_loc, long max_query_len,
                            double scale, long window, long keep_first,
-                           bool sink) {
+                           bool sink, c10::optional<torch::Tensor> sinks,
+                           double softcap) {
   const long T = q.size(0);
   if (T == 0) return;
   const int D = k_cache.size(3);
@@ -398,7 +406,13 @@ void window_attention_mfma(torch::Tensor out, torch::Tensor q,
     gp = gate->data_ptr();
     gs = gate->stride(0);
   }
+  const float *sp = nullptr;
+  if (sinks.has_value()) {
+    TORCH_CHECK(sinks->scalar_type() == at::kFloat && sinks->is_contiguous() &&
+                sinks->numel() == H, "sinks: fp32 [H]");
+    sp = sinks->data_ptr<float>();
+  }
   launch_prefill(out, q, H, D, q.stride(0), k_cache, v_cache, block_table,
                  seq_lens, query_start_loc, max_query_len, scale, window,
-                 keep_first, sink, gp, gs);
+                 keep_first, sink, gp, gs, sp, (float)softcap);
 }

@@ -10,14 +10,22 @@
 //                       pos * f in fp64, so long positions lose
 //                       nothing; pairs (2i, 2i+1) or, half layout,
 //                       (i, i + rot_dims/2)), norm before or after the
-//                       rotation, then q in place and k, v scattered
-//                       into the paged cache (v may be k as projected)
+//                       rotation (or no norm at all), then q in place
+//                       and k, v scattered into the paged cache (v may
+//                       be k as projected; with a value frequency table
+//                       v is turned by its own position over all of Dv)
 //   window_attention    ragged batch (prompt portions beside single
 //                       decode tokens) over the paged cache: position i
 //                       sees j <= i with i - j < window or j < keep_first;
 //                       optional sink: softmax denominator 1 + sum exp(s)
-//                       (a score-0 key with no value); optional fused
-//                       sigmoid output gate
+//                       (a score-0 key with no value) or, with a per-head
+//                       table, exp(sink_h) + sum exp(s); optional tanh cap
+//                       cap * tanh(s / cap) on the scaled scores;
+//                       optional fused sigmoid output gate
+//   rotate_scale_rows   turn the pairs of every head row by sign * pos * f
+//                       and scale (the inverse turn of rotated values)
+//   rms_weight_store    weighted RMS norm of a row, also scattered into a
+//                       single-head paged cache (a low-rank latent)
 //
 // A layer that shares another layer's keys and values calls
 // qk_norm_rope_store with no k/v and attends over the owner's cache.
@@ -41,17 +49,34 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
     const T *__restrict__ k_w, const long *__restrict__ positions,
     const long *__restrict__ slot_mapping, const double *__restrict__ freqs,
     float mag, int rot_dims, T *__restrict__ k_cache, T *__restrict__ v_cache,
-    int H, int G, int D, int Dv, float eps, int half_layout, int norm_last) {
+    int H, int G, int D, int Dv, float eps, int half_layout, int norm_last,
+    int do_norm, const double *__restrict__ v_freqs) {
   extern __shared__ float buf[];
   const int t = blockIdx.x;
   const int y = blockIdx.y;
   const int lane = threadIdx.x;
-  if (y >= H + G) {  // value copy
+  if (y >= H + G) {  // value copy, or value turned by its own position
     const int g = y - H - G;
     const long slot = slot_mapping[t];
     const T *src = v + (long)t * v_stride + (long)g * Dv;
     T *dst = v_cache + (slot * G + g) * Dv;
-    for (int i = lane; i < Dv; i += QK_BLOCK) dst[i] = src[i];
+    if (v_freqs == nullptr) {
+      for (int i = lane; i < Dv; i += QK_BLOCK) dst[i] = src[i];
+      return;
+    }
+    const double vpos = (double)positions[t];
+    const int vhalf = Dv / 2;
+    for (int p = lane; p < vhalf; p += QK_BLOCK) {
+      double sn, cs;
+      sincos(vpos * v_freqs[p], &sn, &cs);
+      const float c = (float)cs, s = (float)sn;
+      const int ia = half_layout ? p : 2 * p;
+      const int ib = half_layout ? p + vhalf : 2 * p + 1;
+      const float a = ScalarOps<T>::to_f32(src[ia]);
+      const float b = ScalarOps<T>::to_f32(src[ib]);
+      dst[ia] = ScalarOps<T>::from_f32(a * c - b * s);
+      dst[ib] = ScalarOps<T>::from_f32(b * c + a * s);
+    }
     return;
   }
   const bool is_q = y < H;
@@ -65,7 +90,7 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
     ss += x * x;
   }
   __syncthreads();
-  if (!norm_last) {
+  if (do_norm && !norm_last) {
     ss = wave_reduce_sum(ss);
     const float inv = 1.0f / sqrtf(ss / D + eps);
     for (int i = lane; i < D; i += QK_BLOCK)
@@ -85,7 +110,7 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
     buf[ib] = b * c + a * s;
   }
   __syncthreads();
-  if (norm_last) {
+  if (do_norm && norm_last) {
     ss = 0.f;
     for (int i = lane; i < D; i += QK_BLOCK) ss += buf[i] * buf[i];
     ss = wave_reduce_sum(ss);
@@ -114,7 +139,8 @@ __global__ __launch_bounds__(ATT_BLOCK) void window_attention_kernel(
     const int *__restrict__ block_table, int bt_stride,
     const int *__restrict__ seq_lens, const int *__restrict__ qsl, int B,
     int H, int G, int D, int Dv, int page, float scale, int window,
-    int keep_first, int sink) {
+    int keep_first, int sink, const float *__restrict__ sinks,
+    float softcap) {
   constexpr int PARTS = ATT_BLOCK / CT;
   constexpr int NC = 2;  // columns per thread when Dv > CT (Dv <= 512)
   extern __shared__ float smem[];
@@ -147,8 +173,10 @@ __global__ __launch_bounds__(ATT_BLOCK) void window_attention_kernel(
   const int n_keep = keep_first < lo ? keep_first : lo;
   const int total = n_keep + (i - lo + 1);
 
-  float m = sink ? 0.f : -INFINITY;
-  float l = sink ? 1.f : 0.f;
+  // the sink is an already-seen key (score 0, or the head's learned
+  // score) that has no value
+  float m = sinks ? sinks[h] : (sink ? 0.f : -INFINITY);
+  float l = (sink || sinks) ? 1.f : 0.f;
   float acc[NC] = {0.f, 0.f};
   const int col = tid % CT, part = tid / CT;
   __syncthreads();
@@ -181,6 +209,7 @@ __global__ __launch_bounds__(ATT_BLOCK) void window_attention_kernel(
           dot += qs[d] * ScalarOps<T>::to_f32(kr[d]);
       }
       s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
     // tile max -> new running max
     float tm = wave_reduce_max(s);
@@ -256,7 +285,8 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
                         c10::optional<torch::Tensor> k_cache,
                         c10::optional<torch::Tensor> v_cache, long H, long G,
                         long D, long Dv, double eps, bool half_layout,
-                        bool norm_last) {
+                        bool norm_last, bool do_norm,
+                        c10::optional<torch::Tensor> v_freqs) {
   const long T = q.size(0);
   if (T == 0) return;
   const auto st = q.scalar_type();
@@ -301,6 +331,13 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
     kcp = k_cache->data_ptr(); vcp = v_cache->data_ptr();
     ks = k->stride(0); vs = v->stride(0);
   }
+  const double *vfp = nullptr;
+  if (v_freqs.has_value()) {
+    TORCH_CHECK(v_freqs->scalar_type() == at::kDouble &&
+                v_freqs->is_contiguous() && Dv % 2 == 0 &&
+                v_freqs->numel() * 2 >= Dv, "value rotary table");
+    vfp = v_freqs->data_ptr<double>();
+  }
   const int gy = own ? H + 2 * G : H;
   auto stream = at::cuda::getCurrentCUDAStream();
 #define RUN(TT)                                                              \
@@ -312,7 +349,8 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
                      own ? slot_mapping.data_ptr<long>() : nullptr,          \
                      freqs.data_ptr<double>(), (float)mag, (int)rot_dims,    \
                      (TT *)kcp, (TT *)vcp, (int)H, (int)G, (int)D, (int)Dv,  \
-                     (float)eps, half_layout ? 1 : 0, norm_last ? 1 : 0)
+                     (float)eps, half_layout ? 1 : 0, norm_last ? 1 : 0,     \
+                     do_norm ? 1 : 0, vfp)
   if (st == at::kBFloat16) RUN(__hip_bfloat16);
   else if (st == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "qk_norm_rope_store: bf16 or fp32");
@@ -325,7 +363,8 @@ void window_attention(torch::Tensor out, torch::Tensor q,
                       torch::Tensor k_cache, torch::Tensor v_cache,
                       torch::Tensor block_table, torch::Tensor seq_lens,
                       torch::Tensor query_start_loc, double scale,
-                      long window, long keep_first, bool sink) {
+                      long window, long keep_first, bool sink,
+                      c10::optional<torch::Tensor> sinks, double softcap) {
   const long T = q.size(0);
   if (T == 0) return;
   const auto st = q.scalar_type();
@@ -337,7 +376,8 @@ void window_attention(torch::Tensor out, torch::Tensor q,
   TORCH_CHECK(H % G == 0, "query heads must be a multiple of kv heads");
   TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
               k_cache.scalar_type() == st && v_cache.scalar_type() == st);
-  TORCH_CHECK(v_cache.size(1) == page && v_cache.size(2) == G);
+  TORCH_CHECK(v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == page &&
+              v_cache.size(2) == G);
   TORCH_CHECK(out.is_contiguous() && out.scalar_type() == st &&
               out.numel() == T * H * Dv);
   TORCH_CHECK(block_table.scalar_type() == at::kInt && block_table.dim() == 2 &&
@@ -356,6 +396,12 @@ void window_attention(torch::Tensor out, torch::Tensor q,
     gp = gate->data_ptr();
     gs = gate->stride(0);
   }
+  const float *sp = nullptr;
+  if (sinks.has_value()) {
+    TORCH_CHECK(sinks->scalar_type() == at::kFloat && sinks->is_contiguous() &&
+                sinks->numel() == H, "sinks: fp32 [H]");
+    sp = sinks->data_ptr<float>();
+  }
   int ct = 16;
   while (ct < Dv && ct < 256) ct *= 2;
   const int parts = ATT_BLOCK / ct;
@@ -373,7 +419,7 @@ void window_attention(torch::Tensor out, torch::Tensor q,
                      seq_lens.data_ptr<int>(),                               \
                      query_start_loc.data_ptr<int>(), B, H, G, D, Dv, page,  \
                      (float)scale, (int)window, (int)keep_first,             \
-                     sink ? 1 : 0)
+                     sink ? 1 : 0, sp, (float)softcap)
 #define RUN_CT(TT)                                                           \
   switch (ct) {                                                              \
     case 16: RUN(TT, 16); break;                                             \
@@ -386,6 +432,134 @@ void window_attention(torch::Tensor out, torch::Tensor q,
   else if (st == at::kFloat) { RUN_CT(float) }
   else TORCH_CHECK(false, "window_attention: bf16 or fp32");
 #undef RUN_CT
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+namespace {
+
+// grid (tokens, heads): turn the pairs of one head row by sign * pos *
+// freqs[m] (pairs (2m, 2m+1), or (m, m + D/2) in the half layout) and
+// scale the result; out may be a column block of a wider buffer.
+template <typename T>
+__global__ __launch_bounds__(QK_BLOCK) void rotate_scale_kernel(
+    T *__restrict__ out, long out_stride, const T *__restrict__ x,
+    long x_stride, const long *__restrict__ positions,
+    const double *__restrict__ freqs, int D, float sign, float scale,
+    int half_layout) {
+  const int t = blockIdx.x, hd = blockIdx.y;
+  const T *src = x + (long)t * x_stride + (long)hd * D;
+  T *dst = out + (long)t * out_stride + (long)hd * D;
+  const double pos = (double)positions[t];
+  const int half = D / 2;
+  for (int p = threadIdx.x; p < half; p += QK_BLOCK) {
+    double sn, cs;
+    sincos(pos * freqs[p], &sn, &cs);
+    const float c = (float)cs, s = sign * (float)sn;
+    const int ia = half_layout ? p : 2 * p;
+    const int ib = half_layout ? p + half : 2 * p + 1;
+    const float a = ScalarOps<T>::to_f32(src[ia]);
+    const float b = ScalarOps<T>::to_f32(src[ib]);
+    dst[ia] = ScalarOps<T>::from_f32((a * c - b * s) * scale);
+    dst[ib] = ScalarOps<T>::from_f32((b * c + a * s) * scale);
+  }
+}
+
+// one wave per row: out = x / rms(x) * w (row kept in the model dtype)
+// and, with a cache, the same row scattered into its paged slot
+template <typename T>
+__global__ __launch_bounds__(ATT_BLOCK) void rms_weight_store_kernel(
+    T *__restrict__ out, const T *__restrict__ x, long x_stride,
+    const T *__restrict__ w, int n, float eps, T *__restrict__ cache,
+    const long *__restrict__ slot_mapping, long rows) {
+  const long r = (long)blockIdx.x * (ATT_BLOCK / WAVE_SIZE) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= rows) return;
+  const T *src = x + r * x_stride;
+  float ss = 0.f;
+  for (int i = lane; i < n; i += WAVE_SIZE) {
+    const float v = ScalarOps<T>::to_f32(src[i]);
+    ss += v * v;
+  }
+  ss = wave_reduce_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / n + eps);
+  T *crow = cache ? cache + slot_mapping[r] * n : nullptr;
+  for (int i = lane; i < n; i += WAVE_SIZE) {
+    const T v = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(src[i]) * inv *
+                                       ScalarOps<T>::to_f32(w[i]));
+    out[r * n + i] = v;
+    if (crow) crow[i] = v;
+  }
+}
+
+}  // namespace
+
+void rotate_scale_rows(torch::Tensor out, torch::Tensor x,
+                       torch::Tensor positions, torch::Tensor freqs,
+                       long heads, long D, double sign, double scale,
+                       bool half_layout) {
+  const long T = x.size(0);
+  if (T == 0) return;
+  const auto st = x.scalar_type();
+  TORCH_CHECK(x.is_cuda() && rows_ok(x) && x.size(1) == heads * D &&
+              D % 2 == 0);
+  TORCH_CHECK(rows_ok(out) && out.size(0) == T && out.size(1) == heads * D &&
+              out.scalar_type() == st);
+  TORCH_CHECK(positions.scalar_type() == at::kLong &&
+              positions.is_contiguous() && positions.numel() >= T);
+  TORCH_CHECK(freqs.scalar_type() == at::kDouble && freqs.is_contiguous() &&
+              freqs.numel() * 2 >= D);
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT)                                                              \
+  hipLaunchKernelGGL((rotate_scale_kernel<TT>), dim3(T, heads),              \
+                     dim3(QK_BLOCK), 0, stream, (TT *)out.data_ptr(),        \
+                     (long)out.stride(0), (const TT *)x.data_ptr(),          \
+                     (long)x.stride(0), positions.data_ptr<long>(),          \
+                     freqs.data_ptr<double>(), (int)D, (float)sign,          \
+                     (float)scale, half_layout ? 1 : 0)
+  if (st == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (st == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "rotate_scale_rows: bf16 or fp32");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+void rms_weight_store(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                      double eps, c10::optional<torch::Tensor> cache,
+                      c10::optional<torch::Tensor> slot_mapping) {
+  const long rows = x.size(0);
+  if (rows == 0) return;
+  const auto st = x.scalar_type();
+  const int n = x.size(1);
+  TORCH_CHECK(x.is_cuda() && rows_ok(x));
+  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == st &&
+              out.numel() == rows * n);
+  TORCH_CHECK(w.scalar_type() == st && w.is_contiguous() && w.numel() == n);
+  void *cp = nullptr;
+  const long *sp = nullptr;
+  if (cache.has_value()) {
+    TORCH_CHECK(slot_mapping.has_value() &&
+                slot_mapping->scalar_type() == at::kLong &&
+                slot_mapping->is_contiguous() &&
+                slot_mapping->numel() >= rows);
+    TORCH_CHECK(cache->is_contiguous() && cache->scalar_type() == st &&
+                cache->size(-1) == n && cache->numel() % n == 0 &&
+                cache->dim() == 4 && cache->size(2) == 1,
+                "latent cache: [pages, page, 1, n]");
+    cp = cache->data_ptr();
+    sp = slot_mapping->data_ptr<long>();
+  }
+  const int per = ATT_BLOCK / WAVE_SIZE;
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT)                                                              \
+  hipLaunchKernelGGL((rms_weight_store_kernel<TT>),                          \
+                     dim3((rows + per - 1) / per), dim3(ATT_BLOCK), 0,       \
+                     stream, (TT *)out.data_ptr(), (const TT *)x.data_ptr(), \
+                     (long)x.stride(0), (const TT *)w.data_ptr(), n,         \
+                     (float)eps, (TT *)cp, sp, rows)
+  if (st == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (st == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "rms_weight_store: bf16 or fp32");
 #undef RUN
   HIP_CHECK_KERNEL();
 }

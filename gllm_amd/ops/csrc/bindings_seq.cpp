@@ -1,7 +1,8 @@
 // Python bindings for the dtype-generic sequence-mixer kernels
-// (gllm_amd._kernels_seq): fp32-residual layer norm, windowed sink
-// attention, talking-heads attention, varlen gated delta rule, plus the
-// grouped MoE GEMM and the activations they are served with.
+// (gllm_amd._kernels_seq): fp32-residual layer norm, hyper-connection
+// streams, windowed sink attention, talking-heads attention, varlen
+// gated delta rule, minGRU, plus the grouped MoE GEMM and the
+// activations they are served with.
 #include <torch/extension.h>
 
 void layernorm_f32(torch::Tensor out, torch::Tensor x, torch::Tensor w,
@@ -22,7 +23,29 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
                         c10::optional<torch::Tensor> k_cache,
                         c10::optional<torch::Tensor> v_cache, long H, long G,
                         long D, long Dv, double eps, bool half_layout,
-                        bool norm_last);
+                        bool norm_last, bool do_norm,
+                        c10::optional<torch::Tensor> v_freqs);
+void rotate_scale_rows(torch::Tensor out, torch::Tensor x,
+                       torch::Tensor positions, torch::Tensor freqs,
+                       long heads, long D, double sign, double scale,
+                       bool half_layout);
+void rms_weight_store(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                      double eps, c10::optional<torch::Tensor> cache,
+                      c10::optional<torch::Tensor> slot_mapping);
+void hyper_streams(torch::Tensor xs, c10::optional<torch::Tensor> y,
+                   c10::optional<torch::Tensor> y2,
+                   c10::optional<torch::Tensor> gate,
+                   c10::optional<torch::Tensor> mix,
+                   c10::optional<torch::Tensor> out_w,
+                   c10::optional<torch::Tensor> h,
+                   c10::optional<torch::Tensor> in_w,
+                   c10::optional<torch::Tensor> g, double eps);
+void mingru_varlen(torch::Tensor out, torch::Tensor zx, torch::Tensor gp,
+                   torch::Tensor state, torch::Tensor slots,
+                   torch::Tensor has_init, torch::Tensor query_start_loc,
+                   double scale, long max_query_len);
+void clamp_swiglu(torch::Tensor out, torch::Tensor x, double limit,
+                  double alpha);
 void talking_attention(torch::Tensor out, torch::Tensor q,
                        torch::Tensor k_cache, torch::Tensor v_cache,
                        torch::Tensor block_table, torch::Tensor seq_lens,
@@ -36,20 +59,24 @@ void window_attention(torch::Tensor out, torch::Tensor q,
                       torch::Tensor k_cache, torch::Tensor v_cache,
                       torch::Tensor block_table, torch::Tensor seq_lens,
                       torch::Tensor query_start_loc, double scale,
-                      long window, long keep_first, bool sink);
+                      long window, long keep_first, bool sink,
+                      c10::optional<torch::Tensor> sinks, double softcap);
 void window_attention_mfma(torch::Tensor out, torch::Tensor q,
                            c10::optional<torch::Tensor> gate,
                            torch::Tensor k_cache, torch::Tensor v_cache,
                            torch::Tensor block_table, torch::Tensor seq_lens,
                            torch::Tensor query_start_loc, long max_query_len,
                            double scale, long window, long keep_first,
-                           bool sink);
+                           bool sink, c10::optional<torch::Tensor> sinks,
+                           double softcap);
 bool window_attention_decode(torch::Tensor out, torch::Tensor q,
                              c10::optional<torch::Tensor> gate,
                              torch::Tensor k_cache, torch::Tensor v_cache,
                              torch::Tensor block_table,
                              torch::Tensor seq_lens, double scale,
-                             long window, long keep_first, bool sink);
+                             long window, long keep_first, bool sink,
+                             c10::optional<torch::Tensor> sinks,
+                             double softcap);
 void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                       torch::Tensor conv_state, torch::Tensor slots,
                       torch::Tensor has_init, torch::Tensor query_start_loc);
@@ -87,6 +114,18 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("talking_attention", &talking_attention,
         "ragged paged causal attention with cross-head score mixing "
         "and a per-head sink");
+  m.def("rotate_scale_rows", &rotate_scale_rows,
+        "turn head-row pairs by sign * position * frequency and scale");
+  m.def("rms_weight_store", &rms_weight_store,
+        "weighted RMS norm of rows, optionally scattered into a paged "
+        "single-head cache");
+  m.def("hyper_streams", &hyper_streams,
+        "multi-stream residual: write a sublayer result back / read the "
+        "next sublayer's scalar-gain RMS-normed input");
+  m.def("mingru_varlen", &mingru_varlen,
+        "ragged minGRU recurrence with a per-slot fp32 state");
+  m.def("clamp_swiglu", &clamp_swiglu,
+        "min(g, limit) * sigmoid(alpha g) * (clamp(u) + 1)");
   m.def("xielu", &xielu, "xIELU activation over row-strided input");
   m.def("relu2", &relu2, "max(x, 0)^2 over row-strided input");
   m.def("window_attention", &window_attention,

@@ -341,3 +341,48 @@ void xielu(torch::Tensor out, torch::Tensor x, double a_pos, double a_neg) {
 void relu2(torch::Tensor out, torch::Tensor x) {
   launch_unary_rows(out, x, Relu2Op{}, "relu2");
 }
+
+namespace {
+
+// out[r, i] = g * sigmoid(alpha g) * (u + 1), g = min(x[r, i], limit),
+// u = clamp(x[r, d + i], -limit, limit); x rows may be strided
+template <typename T>
+__global__ __launch_bounds__(256) void clamp_swiglu_kernel(
+    T *__restrict__ out, const T *__restrict__ x, long x_stride, long rows,
+    int d, float limit, float alpha) {
+  const long total = rows * d;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long r = idx / d;
+    const int i = idx % d;
+    const float g = fminf(ScalarOps<T>::to_f32(x[r * x_stride + i]), limit);
+    const float u = fminf(fmaxf(ScalarOps<T>::to_f32(x[r * x_stride + d + i]),
+                                -limit), limit);
+    out[r * d + i] =
+        ScalarOps<T>::from_f32(g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+  }
+}
+
+}  // namespace
+
+void clamp_swiglu(torch::Tensor out, torch::Tensor x, double limit,
+                  double alpha) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.stride(1) == 1 &&
+              x.size(1) % 2 == 0, "clamp_swiglu: x [rows, 2d] rows");
+  const long rows = x.size(0);
+  const int d = x.size(1) / 2;
+  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == x.scalar_type() &&
+              out.numel() == rows * d);
+  if (rows == 0 || d == 0) return;
+  const int grid = (int)std::min<long>((rows * d + 255) / 256, 65535);
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT)                                                             \
+  hipLaunchKernelGGL((clamp_swiglu_kernel<TT>), dim3(grid), dim3(256), 0,   \
+                     stream, (TT *)out.data_ptr(), (const TT *)x.data_ptr(), \
+                     (long)x.stride(0), rows, d, (float)limit, (float)alpha)
+  if (x.scalar_type() == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (x.scalar_type() == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "clamp_swiglu: bf16 or fp32");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}

@@ -290,12 +290,15 @@ def residual_layernorm(x: torch.Tensor, y: torch.Tensor, w_post, b_post,
 
 def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
                        mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
-                       half_layout=False, norm_last=False):
+                       half_layout=False, norm_last=False, do_norm=True,
+                       v_freqs=None):
     """Per-head RMS norm (plain weight, or none when the weight is None)
     + rotary on q (in place) and k; k, v land in the paged cache rows
     ``slot_mapping``. ``k`` None: a layer that reads another layer's
     cache. ``half_layout``: dimension i pairs with i + rot_dims/2
-    instead of (2i, 2i+1); ``norm_last``: rotate first, then norm."""
+    instead of (2i, 2i+1); ``norm_last``: rotate first, then norm;
+    ``do_norm`` False: rotary only. ``v_freqs`` [Dv/2]: every value row
+    is turned by its own position over all of Dv before it is stored."""
     T = q.shape[0]
     ang = positions[:T].double()[:, None] * freqs.double()[None, :rot_dims // 2]
     cos = (torch.cos(ang).float() * mag)[:, None, :]
@@ -303,6 +306,8 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
     half = rot_dims // 2
 
     def norm(xf, w):
+        if not do_norm:
+            return xf
         xf = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
         return xf if w is None else xf * w.float()
 
@@ -328,14 +333,122 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
     kc = k_cache.view(-1, G, D)
     vc = v_cache.view(-1, G, Dv)
     kc[rows] = prep(k, k_w, G).to(k_cache.dtype)
-    vc[rows] = v.reshape(T, G, Dv).to(v_cache.dtype)
+    vv = v.reshape(T, G, Dv)
+    if v_freqs is not None:
+        vv = rotate_scale_rows(vv.reshape(T, G * Dv), positions, v_freqs,
+                               G, Dv, 1.0, 1.0, half_layout
+                               ).reshape(T, G, Dv)
+    vc[rows] = vv.to(v_cache.dtype)
+
+
+def rotate_scale_rows(x, positions, freqs, heads, D, sign, scale,
+                      half_layout=False, out=None):
+    """Every head row of x [T, heads*D]: pairs (2m, 2m+1) (half
+    layout: (m, m + D/2)) turned by sign * position * freqs[m], then
+    scaled. ``out`` may be a column block of a wider buffer."""
+    T = x.shape[0]
+    half = D // 2
+    ang = positions[:T].double()[:, None] * freqs.double()[None, :half]
+    cos = torch.cos(ang).float()[:, None, :]
+    sin = torch.sin(ang).float()[:, None, :] * sign
+    xf = x.float().reshape(T, heads, D)
+    if half_layout:
+        a, b = xf[..., :half], xf[..., half:]
+        res = torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)
+    else:
+        a, b = xf[..., 0::2], xf[..., 1::2]
+        res = torch.stack([a * cos - b * sin, b * cos + a * sin],
+                          dim=-1).flatten(-2)
+    res = (res * scale).reshape(T, heads * D).to(x.dtype)
+    if out is None:
+        return res
+    out.copy_(res)
+    return out
+
+
+def rms_weight_store(x, w, eps, cache=None, slot_mapping=None):
+    """Weighted RMS norm of rows (fp32 inside, result in x's dtype);
+    with ``cache`` [pages, page, 1, n] the rows also land in their paged
+    slots."""
+    xf = x.float()
+    y = (xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
+         * w.float()).to(x.dtype)
+    if cache is not None:
+        cache.view(-1, x.shape[1])[slot_mapping[:x.shape[0]]] = \
+            y.to(cache.dtype)
+    return y
+
+
+def hyper_streams(xs, y=None, y2=None, gate=None, mix=None, out_w=None,
+                  read=None, dtype=None):
+    """Multi-stream residual xs [S, T, W] fp32. With ``y``: every
+    stream is rewritten from the old ones, x_t = sum_s mix[s, t] x_s +
+    out_w[t] * (y + sigmoid(gate) * y2) (in place). With ``read`` =
+    (in_w [S], gain [1], eps): returns gain * u / rms(u) in ``dtype``,
+    u = sum_s in_w[s] x_s of the (updated) streams."""
+    if y is not None:
+        yv = y.float()
+        if y2 is not None:
+            g = torch.sigmoid(gate.float()) if gate is not None else 1.0
+            yv = yv + g * y2.float()
+        new = torch.einsum("st,snw->tnw", mix.float(), xs) \
+            + out_w.float()[:, None, None] * yv[None]
+        xs.copy_(new)
+    if read is None:
+        return None
+    in_w, gain, eps = read
+    u = torch.einsum("s,snw->nw", in_w.float(), xs)
+    h = u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * gain.float()
+    return h.to(dtype)
+
+
+def mingru_varlen(zx, gp, state, slots, has_init, query_start_loc, scale,
+                  out=None):
+    """Ragged minGRU: zx [T, 2C] = update-gate | candidate
+    pre-activations, gp [T, C] read-out gate; S_t = (1 - z) S_{t-1} +
+    z c with z = sigmoid(zp), c = up + 1/2 (up >= 0) or sigmoid(up);
+    out_t = scale * S_t * silu(gp_t). state [slots, C] fp32 in place."""
+    T, C = gp.shape
+    res = torch.empty(T, C, dtype=torch.float32)
+    qsl = query_start_loc.tolist()
+    z = torch.sigmoid(zx[:, :C].float())
+    up = zx[:, C:].float()
+    cand = torch.where(up >= 0, up + 0.5, torch.sigmoid(up))
+    g = gp.float()
+    g = g * torch.sigmoid(g)
+    st = state.view(-1, C)
+    for b in range(len(qsl) - 1):
+        slot = int(slots[b])
+        S = st[slot].clone() if int(has_init[b]) else torch.zeros(C)
+        for t in range(qsl[b], qsl[b + 1]):
+            S = (1 - z[t]) * S + z[t] * cand[t]
+            res[t] = scale * S * g[t]
+        if qsl[b + 1] > qsl[b]:
+            st[slot] = S
+    res = res.to(zx.dtype)
+    if out is None:
+        return res
+    out.copy_(res)
+    return out
+
+
+def clamp_swiglu(x, limit, alpha):
+    """x [rows, 2d] = gate | up: min(g, limit) * sigmoid(alpha g) *
+    (clamp(u, -limit, limit) + 1)."""
+    d = x.shape[-1] // 2
+    g = x[..., :d].float().clamp(max=limit)
+    u = x[..., d:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1)).to(x.dtype)
 
 
 def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
-                     query_start_loc, scale, window, keep_first, sink):
+                     query_start_loc, scale, window, keep_first, sink,
+                     sinks=None, softcap=0.0):
     """Ragged paged attention: position i sees j <= i with i - j < window
     (window <= 0: all) or j < keep_first; ``sink`` adds 1 to the softmax
-    denominator; ``gate`` multiplies the heads by sigmoid(gate)."""
+    denominator, ``sinks`` [H] adds exp(sinks[h]) instead; ``softcap``:
+    scores become cap * tanh(score / cap); ``gate`` multiplies the heads
+    by sigmoid(gate)."""
     page, G, D = k_cache.shape[1:]
     Dv = v_cache.shape[3]
     T = q.shape[0]
@@ -359,14 +472,22 @@ def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
         kk = kk.repeat_interleave(H // G, dim=1)
         vv = vv.repeat_interleave(H // G, dim=1)
         sc = torch.einsum("ihd,jhd->hij", qf[s:e], kk) * scale
+        if softcap:
+            sc = softcap * torch.tanh(sc / softcap)
         sc = sc.masked_fill(~see[None], float("-inf"))
         m = sc.amax(-1, keepdim=True)
-        if sink:
-            m = m.clamp_min(0.0)
+        if sinks is not None:
+            sk = sinks.float().reshape(H, 1, 1)
+        elif sink:
+            sk = torch.zeros(H, 1, 1)
+        else:
+            sk = None
+        if sk is not None:
+            m = torch.maximum(m, sk)
         p = torch.exp(sc - m)
         den = p.sum(-1, keepdim=True)
-        if sink:
-            den = den + torch.exp(-m)
+        if sk is not None:
+            den = den + torch.exp(sk - m)
         out[s:e] = torch.einsum("hij,jhd->ihd", p / den, vv)
     out = out.reshape(T, H * Dv)
     if gate is not None:

@@ -294,9 +294,14 @@ class ModelRunner:
             self.k_caches = [torch.zeros(
                 (num_pages, spec.page_size, g, dk), dtype=self.kv_dtype,
                 device=self.device) for g, dk, _ in spec.layer_shapes]
+            # value size 0: the layer attends over ONE cached row per
+            # token (a low-rank latent serving as key and value), so
+            # its value cache is the key cache itself
             self.v_caches = [torch.zeros(
                 (num_pages, spec.page_size, g, dv), dtype=self.kv_dtype,
-                device=self.device) for g, _, dv in spec.layer_shapes]
+                device=self.device) if dv else kc
+                for (g, _, dv), kc in zip(spec.layer_shapes,
+                                          self.k_caches)]
             self.idx_caches = None
             return
         self.k_caches = [torch.zeros(kshape, dtype=self.kv_dtype,

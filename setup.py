@@ -32,7 +32,8 @@ HIP_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 CXX_FLAGS = ["-O3", "-std=c++17"]
 
-SEQ_SOURCES = ["bindings_seq.cpp", "layernorm.hip", "attention_window.hip",
+SEQ_SOURCES = ["bindings_seq.cpp", "layernorm.hip", "hyper.hip",
+               "mingru.hip", "attention_window.hip",
                "attention_talking.hip",
                "attention_prefill.hip", "attention_decode.hip",
                "delta_rule.hip", "moe.hip", "elementwise.hip",
