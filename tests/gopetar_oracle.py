@@ -27,11 +27,6 @@ def weight_norm(x, w, eps):
     return rms(x, eps) * w
 
 
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi)
-                                     * (z + 0.044715 * z ** 3)))
-
-
 # ---------------------------------------------------------------- rotary
 def pair_freqs(dims, base):
     i = torch.arange(dims // 2, dtype=F64)
@@ -85,14 +80,15 @@ def window_sink_attention(h, W, p, m):
     k = (h @ W[p + "k"].T + W[p + "k.b"]).reshape(T, G, D)
     v = (h @ W[p + "v"].T + W[p + "v.b"]).reshape(T, G, Dv)
     rot = m.get("rot")
-    if rot and rot["dims"]:
-        f = scaled_freqs(pair_freqs(rot["dims"], rot["base"]),
-                         rot.get("scaling"))
-        q, k = rotate_pairs(q, pos, f), rotate_pairs(k, pos, f)
+    fv = None
+    if rot:
+        if rot.get("dims"):
+            f = scaled_freqs(pair_freqs(rot["dims"], rot["base"]),
+                             rot.get("scaling"))
+            q, k = rotate_pairs(q, pos, f), rotate_pairs(k, pos, f)
+        # the values turn over all of vdim whatever part of q/k does
         fv = pair_freqs(Dv, rot["base"])
         v = rotate_pairs(v, pos, fv)
-    else:
-        fv = None
     out = torch.zeros(T, H, Dv, dtype=F64)
     cap = m.get("softcap")
     win = m["mask"]["size"] if m.get("mask") else 0
