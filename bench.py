@@ -271,11 +271,52 @@ def sudevik_attention_config(sz, vocab=32000):
             "width": sz["width"]}
 
 
+def gopetar_config(sz, vocab=32000, window=4096, streams=2):
+    """Two residual streams; parallel layers (windowed sink attention
+    with rotated values and a tanh cap beside a minGRU as wide as the
+    model) with every fourth layer a latent-attention layer (rank-128
+    latent; the second one reads the first one's cache); MoE with a
+    shared expert in every layer."""
+    H, G, D = sz["attn"]
+    mlp = {"kind": "moe", "expert": {"ff": sz["ff"], "limit": 7.0},
+           "router": {"experts": sz["experts"], "top": sz["top"]},
+           "shared": {"ff": sz["ff"], "limit": 7.0}}
+    layers, first_latent = [], None
+    for i in range(sz["layers"]):
+        if i % 4 == 2:
+            m = {"heads": H, "dim": D, "vdim": D, "kv_rank": 128,
+                 "q_rank": sz["width"] // 2, "scale": D ** -0.5}
+            if first_latent is None:
+                first_latent = i
+            else:
+                m["kv_from"] = first_latent
+            layers.append({"type": "latent_attention", "mlp": mlp,
+                           "mixer": m})
+        else:
+            layers.append({"type": "parallel", "mlp": mlp, "mixer": {
+                "left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D,
+                         "scale": D ** -0.5, "softcap": 30.0,
+                         "mask": {"size": window},
+                         "rot": {"dims": D // 2, "base": 500000.0,
+                                 "scaling": {"factor": 8.0, "low": 1.0,
+                                             "high": 4.0,
+                                             "original": 8192}}},
+                "left_scale": 0.5, "right": {"width": sz["width"]},
+                "right_scale": 0.5}})
+    return {"architecture": "Gopetar", "embedding": {"scale": 1.0},
+            "layers": layers, "norm": {"eps": 1e-5}, "streams": streams,
+            "vocab": vocab, "vocab_size": vocab, "width": sz["width"]}
+
+
 COMPARE_PAIRS = {
     "sudevik": (("sudevik", sudevik_config),
                 ("hybrid-gdn", hybrid_gdn_config)),
     "gukirax": (("gukirax", gukirax_config),
                 ("sudevik-attn", sudevik_attention_config)),
+    # closest existing family: Sudevik (windowed sink attention beside a
+    # recurrent mixer over the state pool, fp32 stream, routed experts)
+    "gopetar": (("gopetar", gopetar_config),
+                ("sudevik", sudevik_config)),
 }
 
 
@@ -287,6 +328,8 @@ MODELS["hybrid-gdn-w2048"] = ("hybrid-GDN-w2048-8L",
                               hybrid_gdn_config(COMPARE_SIZES["w2048"]))
 MODELS["gukirax-w2048"] = ("Gukirax-w2048-8runs",
                            gukirax_config(COMPARE_SIZES["w2048"]))
+MODELS["gopetar-w2048"] = ("Gopetar-w2048-8L",
+                           gopetar_config(COMPARE_SIZES["w2048"]))
 MODELS["sudevik-attn-w2048"] = (
     "Sudevik-attn-w2048-8L",
     sudevik_attention_config(COMPARE_SIZES["w2048"]))
@@ -424,7 +467,9 @@ def main():
                     help="with --mixer-compare: 'sudevik' = Sudevik vs "
                          "hybrid-GDN; 'gukirax' = Gukirax (looped "
                          "talking-heads attention) vs an attention-only "
-                         "Sudevik stack of as many layer runs")
+                         "Sudevik stack of as many layer runs; 'gopetar' "
+                         "= Gopetar (two streams, attention beside a "
+                         "minGRU, latent attention) vs Sudevik")
     ap.add_argument("--compare-sizes", type=str, default="w2048,w1024")
     ap.add_argument("--compare-decode", type=str, default="1,32,128")
     ap.add_argument("--compare-prefill-batch", type=int, default=4)

@@ -33,13 +33,16 @@ void window_attention_mfma(torch::Tensor out, torch::Tensor q,
                            torch::Tensor block_table, torch::Tensor seq_lens,
                            torch::Tensor query_start_loc, long max_query_len,
                            double scale, long window, long keep_first,
-                           bool sink);
+                           bool sink, c10::optional<torch::Tensor> sinks,
+                           double softcap);
 bool window_attention_decode(torch::Tensor out, torch::Tensor q,
                              c10::optional<torch::Tensor> gate,
                              torch::Tensor k_cache, torch::Tensor v_cache,
                              torch::Tensor block_table,
                              torch::Tensor seq_lens, double scale,
-                             long window, long keep_first, bool sink);
+                             long window, long keep_first, bool sink,
+                             c10::optional<torch::Tensor> sinks,
+                             double softcap);
 void mla_paged_attention(torch::Tensor out, torch::Tensor q,
                          torch::Tensor k_cache, torch::Tensor block_table,
                          torch::Tensor seq_lens,

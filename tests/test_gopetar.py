@@ -169,6 +169,29 @@ STACK = [latent(mlp=moe_ff()),
                   rot_dims=10, softcap=0, gru=13, mlp=moe_ff(top=3))]
 
 
+def stack_for(dtype, layers=None):
+    """fp32 runs route for real. In bf16 the 16-bit rounding of a
+    router's input flips a close top-k call now and then, and here a
+    flip does not stay at its position: it changes keys, latents and the
+    recurrent state that every later position reads. So the multi-layer
+    bf16 runs use every expert (top = experts: the grouped GEMM, the
+    routing weights and their softmax still run, nothing discrete is
+    left); discrete routing in bf16 is covered by the one-layer models
+    of test_each_mechanism_alone, where a flip stays local."""
+    layers = STACK if layers is None else layers
+    if dtype != "bfloat16":
+        return layers
+    out = []
+    for lay in layers:
+        if lay.get("mlp"):
+            mlp = dict(lay["mlp"])
+            mlp["router"] = dict(mlp["router"],
+                                 top=mlp["router"]["experts"])
+            lay = dict(lay, mlp=mlp)
+        out.append(lay)
+    return out
+
+
 # ------------------------------------------------------------------ harness
 def engine(model_dir, device, dtype, max_tokens=256, slots=4, page=16):
     from gllm_amd.entrypoints.trace_replay import build_engine
@@ -297,7 +320,7 @@ def test_each_mechanism_alone(name, device, dtype, width):
 def test_layer_trail_matches(device, dtype):
     """The summed streams after every layer against the oracle's,
     through the model's layer probe."""
-    cfg = make_config(STACK, width=40, vocab=90, streams=3)
+    cfg = make_config(stack_for(dtype), width=40, vocab=90, streams=3)
     w = make_weights(cfg, 21)
     llm = engine(save_model(cfg, w), device, dtype)
     toks = tokens_for(cfg, 19, 22)
@@ -320,7 +343,7 @@ def test_prefill_decode_and_portions(device, dtype):
     windows (9 and 17 keys) are crossed inside portions, at their starts
     and by decoded tokens; the recurrent state is handed from portion to
     portion."""
-    cfg = make_config(STACK, width=40, vocab=90, streams=3)
+    cfg = make_config(stack_for(dtype), width=40, vocab=90, streams=3)
     w = make_weights(cfg, 3)
     llm = engine(save_model(cfg, w), device, dtype)
     toks = tokens_for(cfg, 61, 4)
@@ -343,7 +366,7 @@ def test_mixed_batches_recycle_pages_and_slots(device, dtype):
     tokens) equal each request alone; the pool holds 10 pages and 3
     state slots, so later requests land on freed pages and on slots
     that still hold another sequence's state."""
-    cfg = make_config(STACK, width=32, vocab=64, streams=2)
+    cfg = make_config(stack_for(dtype), width=32, vocab=64, streams=2)
     w = make_weights(cfg, 5)
     llm = engine(save_model(cfg, w), device, dtype, max_tokens=160, slots=3)
     P = {c: tokens_for(cfg, n, 10 + i)
@@ -401,13 +424,12 @@ def test_long_decoding(device, dtype):
     """A short prompt, then 150 tokens decoded one by one: ten pages of
     context grow under the decode path, the windows slide over decoded
     tokens only, the state is carried 150 times; every position."""
-    cfg = make_config(
-        [parallel(heads=4, kv_heads=2, dim=8, vdim=8, window=33,
-                  mlp=moe_ff()),
-         latent(mlp=moe_ff(experts=3, top=2, shared=0)),
-         parallel(heads=2, kv_heads=1, dim=16, vdim=4, rot_dims=6,
-                  window=16, gru=9)],
-        width=24, vocab=40, streams=2)
+    cfg = make_config(stack_for(dtype, [
+        parallel(heads=4, kv_heads=2, dim=8, vdim=8, window=33,
+                 mlp=moe_ff()),
+        latent(mlp=moe_ff(experts=3, top=2, shared=0)),
+        parallel(heads=2, kv_heads=1, dim=16, vdim=4, rot_dims=6,
+                 window=16, gru=9)]), width=24, vocab=40, streams=2)
     w = make_weights(cfg, 9)
     llm = engine(save_model(cfg, w), device, dtype)
     toks = tokens_for(cfg, 156, 11)
@@ -685,7 +707,7 @@ def test_greedy_generation_through_the_scheduler(device, dtype):
     from gllm_amd.config import EngineConfig
     from gllm_amd.engine.llm import LLM
     from gllm_amd.sequence import SamplingParams
-    cfg = make_config(STACK, width=32, vocab=48, streams=2)
+    cfg = make_config(stack_for(dtype), width=32, vocab=48, streams=2)
     w = make_weights(cfg, 14)
     d = save_model(cfg, w)
     config = EngineConfig(model=d, dtype=dtype, device=device, page_size=16,
