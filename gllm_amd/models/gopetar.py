@@ -249,8 +249,6 @@ class GopetarLayer(nn.Module):
 class GopetarForCausalLM(nn.Module):
     # the ragged state kernel reads slots / flags from device tensors
     wants_state_tensors = True
-    # the eager path serves; decode buckets are not captured
-    supports_graph = False
 
     def __init__(self, cfg, engine_config):
         super().__init__()
@@ -325,6 +323,14 @@ class GopetarForCausalLM(nn.Module):
         # the last read: plain sum of the streams through the final norm
         self.final = sum_reader(self.streams, eps)
         self.lm_head = ParallelLMHead(vocab, width, params_dtype=dtype)
+        # hipGraph decode buckets need a sync-free forward: bf16 with
+        # every MoE on the grouped GEMM (8-aligned width and ff); fp32
+        # and odd expert shapes take the host segment loop
+        self.supports_graph = dtype == torch.bfloat16 and all(
+            lay.mlp is None or (width % 8 == 0 and
+                                lay.mlp.experts.intermediate_per_rank % 8
+                                == 0)
+            for lay in mods)
         # called as layer_probe(layer index, summed stream) after a layer
         self.layer_probe = None
 

@@ -438,26 +438,55 @@ void window_attention(torch::Tensor out, torch::Tensor q,
 
 namespace {
 
-// grid (tokens, heads): turn the pairs of one head row by sign * pos *
-// freqs[m] (pairs (2m, 2m+1), or (m, m + D/2) in the half layout) and
-// scale the result; out may be a column block of a wider buffer.
+// one workgroup per token: the cos/sin of the token's D/2 pair angles
+// (sign * pos * freqs[m], fp64 angle) are formed once in LDS, then every
+// head row is turned (pairs (2m, 2m+1), or (m, m + D/2) in the half
+// layout) and scaled; out may be a column block of a wider buffer.
 template <typename T>
-__global__ __launch_bounds__(QK_BLOCK) void rotate_scale_kernel(
+__global__ __launch_bounds__(ATT_BLOCK) void rotate_scale_kernel(
     T *__restrict__ out, long out_stride, const T *__restrict__ x,
     long x_stride, const long *__restrict__ positions,
-    const double *__restrict__ freqs, int D, float sign, float scale,
-    int half_layout) {
-  const int t = blockIdx.x, hd = blockIdx.y;
-  const T *src = x + (long)t * x_stride + (long)hd * D;
-  T *dst = out + (long)t * out_stride + (long)hd * D;
-  const double pos = (double)positions[t];
+    const double *__restrict__ freqs, int heads, int D, float sign,
+    float scale, int layout) {
+  // layout 0: pairs (2m, 2m+1) moved as 32-bit words; 1: pairs
+  // (m, m + D/2); 2: pairs (2m, 2m+1) element by element
+  const bool half_layout = layout == 1;
+  extern __shared__ float cs_tab[];  // [D/2] cos, [D/2] sin
+  const int t = blockIdx.x;
   const int half = D / 2;
-  for (int p = threadIdx.x; p < half; p += QK_BLOCK) {
+  const double pos = (double)positions[t];
+  for (int p = threadIdx.x; p < half; p += ATT_BLOCK) {
     double sn, cs;
     sincos(pos * freqs[p], &sn, &cs);
-    const float c = (float)cs, s = sign * (float)sn;
-    const int ia = half_layout ? p : 2 * p;
-    const int ib = half_layout ? p + half : 2 * p + 1;
+    cs_tab[p] = (float)cs;
+    cs_tab[half + p] = sign * (float)sn;
+  }
+  __syncthreads();
+  const T *src = x + (long)t * x_stride;
+  T *dst = out + (long)t * out_stride;
+  const int total = heads * half;
+  if (layout == 0 && sizeof(T) == 2) {
+    // a pair is one aligned 32-bit word of the row
+    for (int idx = threadIdx.x; idx < total; idx += ATT_BLOCK) {
+      const int p = idx % half;
+      const float c = cs_tab[p], s = cs_tab[half + p];
+      T pr[2];
+      *reinterpret_cast<unsigned *>(pr) =
+          reinterpret_cast<const unsigned *>(src)[idx];
+      const float a = ScalarOps<T>::to_f32(pr[0]);
+      const float b = ScalarOps<T>::to_f32(pr[1]);
+      pr[0] = ScalarOps<T>::from_f32((a * c - b * s) * scale);
+      pr[1] = ScalarOps<T>::from_f32((b * c + a * s) * scale);
+      reinterpret_cast<unsigned *>(dst)[idx] =
+          *reinterpret_cast<unsigned *>(pr);
+    }
+    return;
+  }
+  for (int idx = threadIdx.x; idx < total; idx += ATT_BLOCK) {
+    const int hd = idx / half, p = idx % half;
+    const float c = cs_tab[p], s = cs_tab[half + p];
+    const int ia = hd * D + (half_layout ? p : 2 * p);
+    const int ib = hd * D + (half_layout ? p + half : 2 * p + 1);
     const float a = ScalarOps<T>::to_f32(src[ia]);
     const float b = ScalarOps<T>::to_f32(src[ib]);
     dst[ia] = ScalarOps<T>::from_f32((a * c - b * s) * scale);
@@ -510,13 +539,19 @@ void rotate_scale_rows(torch::Tensor out, torch::Tensor x,
   TORCH_CHECK(freqs.scalar_type() == at::kDouble && freqs.is_contiguous() &&
               freqs.numel() * 2 >= D);
   auto stream = at::cuda::getCurrentCUDAStream();
+  // the word-wide path needs 4-byte aligned rows on both sides
+  const bool words = x.element_size() == 2 &&
+                     reinterpret_cast<uintptr_t>(x.data_ptr()) % 4 == 0 &&
+                     reinterpret_cast<uintptr_t>(out.data_ptr()) % 4 == 0 &&
+                     x.stride(0) % 2 == 0 && out.stride(0) % 2 == 0;
+  const int layout = half_layout ? 1 : (words ? 0 : 2);
 #define RUN(TT)                                                              \
-  hipLaunchKernelGGL((rotate_scale_kernel<TT>), dim3(T, heads),              \
-                     dim3(QK_BLOCK), 0, stream, (TT *)out.data_ptr(),        \
+  hipLaunchKernelGGL((rotate_scale_kernel<TT>), dim3(T), dim3(ATT_BLOCK),    \
+                     D * sizeof(float), stream, (TT *)out.data_ptr(),        \
                      (long)out.stride(0), (const TT *)x.data_ptr(),          \
                      (long)x.stride(0), positions.data_ptr<long>(),          \
-                     freqs.data_ptr<double>(), (int)D, (float)sign,          \
-                     (float)scale, half_layout ? 1 : 0)
+                     freqs.data_ptr<double>(), (int)heads, (int)D,           \
+                     (float)sign, (float)scale, layout)
   if (st == at::kBFloat16) RUN(__hip_bfloat16);
   else if (st == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "rotate_scale_rows: bf16 or fp32");

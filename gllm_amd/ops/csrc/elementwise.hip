@@ -345,11 +345,34 @@ void relu2(torch::Tensor out, torch::Tensor x) {
 namespace {
 
 // out[r, i] = g * sigmoid(alpha g) * (u + 1), g = min(x[r, i], limit),
-// u = clamp(x[r, d + i], -limit, limit); x rows may be strided
-template <typename T>
+// u = clamp(x[r, d + i], -limit, limit); x rows may be strided. VEC: 8
+// elements per thread through 16 B accesses (d % 8 == 0, aligned rows).
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void clamp_swiglu_kernel(
     T *__restrict__ out, const T *__restrict__ x, long x_stride, long rows,
     int d, float limit, float alpha) {
+  if (VEC) {
+    const int nvec = d / 8;
+    const long total = rows * nvec;
+    for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+      const long r = idx / nvec;
+      const int i = (idx % nvec) * 8;
+      float g[8], u[8];
+      ld8<T>(x + r * x_stride + i, g);
+      ld8<T>(x + r * x_stride + d + i, u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float gv = fminf(g[e], limit);
+        const float uv = fminf(fmaxf(u[e], -limit), limit);
+        g[e] = gv / (1.0f + (sizeof(T) == 4 ? expf(-alpha * gv)
+                                            : __expf(-alpha * gv))) *
+               (uv + 1.0f);
+      }
+      st8<T>(out + r * d + i, g);
+    }
+    return;
+  }
   const long total = rows * d;
   for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
        idx += (long)gridDim.x * blockDim.x) {
@@ -374,15 +397,26 @@ void clamp_swiglu(torch::Tensor out, torch::Tensor x, double limit,
   TORCH_CHECK(out.is_contiguous() && out.scalar_type() == x.scalar_type() &&
               out.numel() == rows * d);
   if (rows == 0 || d == 0) return;
-  const int grid = (int)std::min<long>((rows * d + 255) / 256, 65535);
+  const long esz = x.element_size();
+  const bool vec = d % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0 &&
+                   (x.stride(0) * esz) % 16 == 0;
+  const long work = vec ? rows * (d / 8) : rows * (long)d;
+  const int grid = (int)std::min<long>((work + 255) / 256, 8192);
   auto stream = at::cuda::getCurrentCUDAStream();
-#define RUN(TT)                                                             \
-  hipLaunchKernelGGL((clamp_swiglu_kernel<TT>), dim3(grid), dim3(256), 0,   \
-                     stream, (TT *)out.data_ptr(), (const TT *)x.data_ptr(), \
-                     (long)x.stride(0), rows, d, (float)limit, (float)alpha)
-  if (x.scalar_type() == at::kBFloat16) RUN(__hip_bfloat16);
-  else if (x.scalar_type() == at::kFloat) RUN(float);
-  else TORCH_CHECK(false, "clamp_swiglu: bf16 or fp32");
+#define RUN(TT, V)                                                          \
+  hipLaunchKernelGGL((clamp_swiglu_kernel<TT, V>), dim3(grid), dim3(256),   \
+                     0, stream, (TT *)out.data_ptr(),                       \
+                     (const TT *)x.data_ptr(), (long)x.stride(0), rows, d,  \
+                     (float)limit, (float)alpha)
+  if (x.scalar_type() == at::kBFloat16) {
+    if (vec) RUN(__hip_bfloat16, true); else RUN(__hip_bfloat16, false);
+  } else if (x.scalar_type() == at::kFloat) {
+    if (vec) RUN(float, true); else RUN(float, false);
+  } else {
+    TORCH_CHECK(false, "clamp_swiglu: bf16 or fp32");
+  }
 #undef RUN
   HIP_CHECK_KERNEL();
 }

@@ -26,7 +26,31 @@ namespace {
 constexpr int HY_BLOCK = 256;
 constexpr int MAX_S = 8;
 
-template <typename T>
+// 4 consecutive elements <-> fp32 (8 B for 16-bit types, 16 B for fp32)
+template <typename T> DEV_INLINE void ld4(const T *p, float *f) {
+  const shortx4 v = *reinterpret_cast<const shortx4 *>(p);
+  const T *e = reinterpret_cast<const T *>(&v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[i] = ScalarOps<T>::to_f32(e[i]);
+}
+template <> DEV_INLINE void ld4<float>(const float *p, float *f) {
+  const floatx4 v = *reinterpret_cast<const floatx4 *>(p);
+  f[0] = v[0]; f[1] = v[1]; f[2] = v[2]; f[3] = v[3];
+}
+template <typename T> DEV_INLINE void st4(T *p, const float *f) {
+  shortx4 v;
+  T *e = reinterpret_cast<T *>(&v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) e[i] = ScalarOps<T>::from_f32(f[i]);
+  *reinterpret_cast<shortx4 *>(p) = v;
+}
+template <> DEV_INLINE void st4<float>(float *p, const float *f) {
+  *reinterpret_cast<floatx4 *>(p) = floatx4{f[0], f[1], f[2], f[3]};
+}
+
+// V = 4: four columns per thread through 8 / 16 B accesses (W % 4 == 0,
+// aligned rows); V = 1: element by element.
+template <typename T, int V>
 __global__ __launch_bounds__(HY_BLOCK) void hyper_kernel(
     float *__restrict__ xs, long stream_stride, int S, int W,
     // write part (y == nullptr: read only)
@@ -54,41 +78,74 @@ __global__ __launch_bounds__(HY_BLOCK) void hyper_kernel(
     gy = 1.0f / (1.0f + expf(-z));
   }
   float ss = 0.f;
-  for (int c = tid; c < W; c += HY_BLOCK) {
-    float old[MAX_S];
+  for (int c = tid * V; c < W; c += HY_BLOCK * V) {
+    float old[MAX_S][V];
 #pragma unroll
     for (int s = 0; s < MAX_S; ++s)
-      if (s < S) old[s] = xs[s * stream_stride + t * W + c];
-    float u = 0.f;
+      if (s < S) {
+        if (V == 4) ld4<float>(xs + s * stream_stride + t * W + c, old[s]);
+        else old[s][0] = xs[s * stream_stride + t * W + c];
+      }
+    float u[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) u[e] = 0.f;
     if (y != nullptr) {
-      float yv = ScalarOps<T>::to_f32(y[t * y_stride + c]);
-      if (y2 != nullptr)
-        yv += gy * ScalarOps<T>::to_f32(y2[t * y2_stride + c]);
+      float yv[V];
+      if (V == 4) ld4<T>(y + t * y_stride + c, yv);
+      else yv[0] = ScalarOps<T>::to_f32(y[t * y_stride + c]);
+      if (y2 != nullptr) {
+        float y2v[V];
+        if (V == 4) ld4<T>(y2 + t * y2_stride + c, y2v);
+        else y2v[0] = ScalarOps<T>::to_f32(y2[t * y2_stride + c]);
+#pragma unroll
+        for (int e = 0; e < V; ++e) yv[e] += gy * y2v[e];
+      }
 #pragma unroll
       for (int to = 0; to < MAX_S; ++to) {
         if (to >= S) break;
-        float nv = b_s[to] * yv;
+        float nv[V];
+#pragma unroll
+        for (int e = 0; e < V; ++e) nv[e] = b_s[to] * yv[e];
 #pragma unroll
         for (int s = 0; s < MAX_S; ++s)
-          if (s < S) nv += m_s[s * S + to] * old[s];
-        xs[to * stream_stride + t * W + c] = nv;
-        u += a_s[to] * nv;
+          if (s < S) {
+#pragma unroll
+            for (int e = 0; e < V; ++e) nv[e] += m_s[s * S + to] * old[s][e];
+          }
+        if (V == 4) st4<float>(xs + to * stream_stride + t * W + c, nv);
+        else xs[to * stream_stride + t * W + c] = nv[0];
+#pragma unroll
+        for (int e = 0; e < V; ++e) u[e] += a_s[to] * nv[e];
       }
     } else {
 #pragma unroll
       for (int s = 0; s < MAX_S; ++s)
-        if (s < S) u += a_s[s] * old[s];
+        if (s < S) {
+#pragma unroll
+          for (int e = 0; e < V; ++e) u[e] += a_s[s] * old[s][e];
+        }
     }
     if (h != nullptr) {
-      u_row[c] = u;
-      ss += u * u;
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        u_row[c + e] = u[e];
+        ss += u[e] * u[e];
+      }
     }
   }
   if (h == nullptr) return;
   ss = block_reduce_sum<HY_BLOCK>(ss, red);
   const float k = g[0] / sqrtf(ss / W + eps);
-  for (int c = tid; c < W; c += HY_BLOCK)
-    h[t * W + c] = ScalarOps<T>::from_f32(u_row[c] * k);
+  for (int c = tid * V; c < W; c += HY_BLOCK * V) {
+    if (V == 4) {
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = u_row[c + e] * k;
+      st4<T>(h + t * W + c, o);
+    } else {
+      h[t * W + c] = ScalarOps<T>::from_f32(u_row[c] * k);
+    }
+  }
 }
 
 const float *f32_vec(const c10::optional<torch::Tensor> &t, long n,
@@ -118,7 +175,8 @@ void hyper_streams(torch::Tensor xs, c10::optional<torch::Tensor> y,
   const long T = xs.size(1);
   if (T == 0) return;
   TORCH_CHECK(S >= 1 && S <= MAX_S, "1..", MAX_S, " streams");
-  TORCH_CHECK((size_t)W * sizeof(float) <= 96 * 1024, "row too wide");
+  TORCH_CHECK((size_t)W * sizeof(float) <= 64 * 1024,
+              "row wider than the 64 KB of LDS a launch gets by default");
   TORCH_CHECK(y.has_value() || h.has_value());
   auto st = y.has_value() ? y->scalar_type() : h->scalar_type();
   const void *yp = nullptr, *y2p = nullptr, *gp = nullptr;
@@ -153,15 +211,30 @@ void hyper_streams(torch::Tensor xs, c10::optional<torch::Tensor> y,
     gnp = f32_vec(g, 1, "norm gain");
   }
   auto stream = at::cuda::getCurrentCUDAStream();
-#define RUN(TT)                                                             \
-  hipLaunchKernelGGL((hyper_kernel<TT>), dim3(T), dim3(HY_BLOCK),           \
+  // four columns per thread when every row is 16 B (fp32) / 8 B (16-bit)
+  // aligned
+  const long esz = st == at::kFloat ? 4 : 2;
+  auto row_ok = [&](const void *p, long stride) {
+    return p == nullptr ||
+           (reinterpret_cast<uintptr_t>(p) % (4 * esz) == 0 &&
+            (stride * esz) % (4 * esz) == 0);
+  };
+  const bool vec = W % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(xs.data_ptr()) % 16 == 0 &&
+                   row_ok(yp, ys) && row_ok(y2p, y2s) && row_ok(hp, W);
+#define RUN(TT, V)                                                          \
+  hipLaunchKernelGGL((hyper_kernel<TT, V>), dim3(T), dim3(HY_BLOCK),        \
                      W * sizeof(float), stream, xs.data_ptr<float>(),       \
                      (long)xs.stride(0), S, W, (const TT *)yp, ys,          \
                      (const TT *)y2p, y2s, (const TT *)gp, gs, mp, bp,      \
                      (TT *)hp, ap, gnp, (float)eps)
-  if (st == at::kBFloat16) RUN(__hip_bfloat16);
-  else if (st == at::kFloat) RUN(float);
-  else TORCH_CHECK(false, "hyper_streams: bf16 or fp32");
+  if (st == at::kBFloat16) {
+    if (vec) RUN(__hip_bfloat16, 4); else RUN(__hip_bfloat16, 1);
+  } else if (st == at::kFloat) {
+    if (vec) RUN(float, 4); else RUN(float, 1);
+  } else {
+    TORCH_CHECK(false, "hyper_streams: bf16 or fp32");
+  }
 #undef RUN
   HIP_CHECK_KERNEL();
 }

@@ -700,10 +700,15 @@ def test_hyper_streams_op(device, dtype):
             assert (h2.float() - h.float()).abs().max() < tol
 
 
+@pytest.mark.parametrize("graph", [False, True], ids=["eager", "graph"])
 @pytest.mark.parametrize("device,dtype", DEVICES)
-def test_greedy_generation_through_the_scheduler(device, dtype):
+def test_greedy_generation_through_the_scheduler(device, dtype, graph):
     """LLM.generate (scheduler policy, chunked prefill, sampler) picks
-    the oracle's greedy tokens."""
+    the oracle's greedy tokens; with ``graph`` the decode steps replay
+    captured hipGraph buckets (bf16 on the GPU only), interleaved with
+    the eager prefill steps of the later prompts."""
+    if graph and (device, dtype) != ("cuda", "bfloat16"):
+        pytest.skip("decode graphs are captured for bf16 on the GPU")
     from gllm_amd.config import EngineConfig
     from gllm_amd.engine.llm import LLM
     from gllm_amd.sequence import SamplingParams
@@ -711,9 +716,10 @@ def test_greedy_generation_through_the_scheduler(device, dtype):
     w = make_weights(cfg, 14)
     d = save_model(cfg, w)
     config = EngineConfig(model=d, dtype=dtype, device=device, page_size=16,
-                          maxp=16, maxd=8, use_graph=False,
+                          maxp=16, maxd=8, use_graph=graph, max_graph_bs=8,
                           model_max_length=256, enable_overlap=False)
     llm = LLM(config=config, num_pages_override=64)
+    assert (llm.runner.graph_runner is not None) == graph
     prompts = [tokens_for(cfg, n, 20 + n) for n in (5, 37, 18)]
     outs = llm.generate(prompts, SamplingParams(
         temperature=0.0, max_tokens=12, ignore_eos=True))
