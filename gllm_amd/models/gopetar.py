@@ -186,10 +186,13 @@ class ClampedExperts(nn.Module):
         self.shared_ff = int(_get(shared, "ff")) if shared else 0
         if self.shared_ff:
             self.shared_limit = float(_get(shared, "limit"))
-            # gate rows | up rows | the one-row result gate
-            self.sizes = [self.shared_ff, self.shared_ff, 1]
+            # gate rows | up rows | the one-row result gate, padded with
+            # zero rows to 8 so that the rows of the projection's output
+            # stay 16 B aligned for the activation kernel
+            self.sizes = [self.shared_ff, self.shared_ff, 8]
             self.shared_in = MergedColumnParallelLinear(
                 width, self.sizes, params_dtype=dtype)
+            self.shared_in.weight.data.zero_()
             self.shared_down = RowParallelLinear(self.shared_ff, width,
                                                  params_dtype=dtype)
         self._r32 = None
@@ -205,7 +208,8 @@ class ClampedExperts(nn.Module):
         proj = self.shared_in(h)
         act = ops.clamp_swiglu(proj[:, :2 * self.shared_ff],
                                self.shared_limit, EXPERT_ALPHA)
-        return y, self.shared_down(act), proj[:, 2 * self.shared_ff:]
+        return y, self.shared_down(act), \
+            proj[:, 2 * self.shared_ff:2 * self.shared_ff + 1]
 
 
 class GopetarLayer(nn.Module):
@@ -470,7 +474,11 @@ class GopetarForCausalLM(nn.Module):
             if sub[1] == "down":
                 self._copy(mlp.shared_down.weight, w)
                 return True
-            shard = {"gate": 0, "up": 1, "sg": 2}.get(sub[1])
+            if sub[1] == "sg":
+                self._copy(mlp.shared_in.weight.data[
+                    2 * mlp.shared_ff:2 * mlp.shared_ff + 1], w)
+                return True
+            shard = {"gate": 0, "up": 1}.get(sub[1])
             if shard is None:
                 return False
             p = mlp.shared_in.weight

@@ -495,8 +495,9 @@ __global__ __launch_bounds__(ATT_BLOCK) void rotate_scale_kernel(
 }
 
 // one wave per row: out = x / rms(x) * w (row kept in the model dtype)
-// and, with a cache, the same row scattered into its paged slot
-template <typename T>
+// and, with a cache, the same row scattered into its paged slot. VEC: 8
+// elements per lane through 16 B accesses (n % 8 == 0, aligned rows).
+template <typename T, bool VEC>
 __global__ __launch_bounds__(ATT_BLOCK) void rms_weight_store_kernel(
     T *__restrict__ out, const T *__restrict__ x, long x_stride,
     const T *__restrict__ w, int n, float eps, T *__restrict__ cache,
@@ -505,14 +506,34 @@ __global__ __launch_bounds__(ATT_BLOCK) void rms_weight_store_kernel(
   const int lane = threadIdx.x & 63;
   if (r >= rows) return;
   const T *src = x + r * x_stride;
+  T *crow = cache ? cache + slot_mapping[r] * n : nullptr;
   float ss = 0.f;
+  if (VEC) {
+    for (int i = lane * 8; i < n; i += WAVE_SIZE * 8) {
+      float f[8];
+      ld8<T>(src + i, f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+    }
+    ss = wave_reduce_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / n + eps);
+    for (int i = lane * 8; i < n; i += WAVE_SIZE * 8) {
+      float f[8], wf[8];
+      ld8<T>(src + i, f);
+      ld8<T>(w + i, wf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = f[e] * inv * wf[e];
+      st8<T>(out + r * n + i, f);
+      if (crow) st8<T>(crow + i, f);
+    }
+    return;
+  }
   for (int i = lane; i < n; i += WAVE_SIZE) {
     const float v = ScalarOps<T>::to_f32(src[i]);
     ss += v * v;
   }
   ss = wave_reduce_sum(ss);
   const float inv = 1.0f / sqrtf(ss / n + eps);
-  T *crow = cache ? cache + slot_mapping[r] * n : nullptr;
   for (int i = lane; i < n; i += WAVE_SIZE) {
     const T v = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(src[i]) * inv *
                                        ScalarOps<T>::to_f32(w[i]));
@@ -586,15 +607,26 @@ void rms_weight_store(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   }
   const int per = ATT_BLOCK / WAVE_SIZE;
   auto stream = at::cuda::getCurrentCUDAStream();
-#define RUN(TT)                                                              \
-  hipLaunchKernelGGL((rms_weight_store_kernel<TT>),                          \
+  const long esz = x.element_size();
+  auto al16 = [](const void *p) {
+    return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0;
+  };
+  const bool vec = n % 8 == 0 && (x.stride(0) * esz) % 16 == 0 &&
+                   al16(x.data_ptr()) && al16(out.data_ptr()) &&
+                   al16(w.data_ptr()) && al16(cp);
+#define RUN(TT, V)                                                           \
+  hipLaunchKernelGGL((rms_weight_store_kernel<TT, V>),                       \
                      dim3((rows + per - 1) / per), dim3(ATT_BLOCK), 0,       \
                      stream, (TT *)out.data_ptr(), (const TT *)x.data_ptr(), \
                      (long)x.stride(0), (const TT *)w.data_ptr(), n,         \
                      (float)eps, (TT *)cp, sp, rows)
-  if (st == at::kBFloat16) RUN(__hip_bfloat16);
-  else if (st == at::kFloat) RUN(float);
-  else TORCH_CHECK(false, "rms_weight_store: bf16 or fp32");
+  if (st == at::kBFloat16) {
+    if (vec) RUN(__hip_bfloat16, true); else RUN(__hip_bfloat16, false);
+  } else if (st == at::kFloat) {
+    if (vec) RUN(float, true); else RUN(float, false);
+  } else {
+    TORCH_CHECK(false, "rms_weight_store: bf16 or fp32");
+  }
 #undef RUN
   HIP_CHECK_KERNEL();
 }

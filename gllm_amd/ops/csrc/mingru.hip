@@ -61,6 +61,7 @@ __global__ __launch_bounds__(CH *NSEG) void mingru_kernel(
   if (NSEG > 1) {
     float A = 1.f, B = 0.f;
     if (live)
+#pragma unroll 4
       for (int t = lo; t < hi; ++t) {
         float a, bb;
         gru_step<T>(zx + (long)t * zx_stride, C, c, a, bb);
@@ -73,6 +74,7 @@ __global__ __launch_bounds__(CH *NSEG) void mingru_kernel(
     for (int s = 0; s < seg; ++s) S = fa[s][cx] * S + fb[s][cx];
   }
   if (!live) return;
+#pragma unroll 4
   for (int t = lo; t < hi; ++t) {
     float a, bb;
     gru_step<T>(zx + (long)t * zx_stride, C, c, a, bb);
