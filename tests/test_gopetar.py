@@ -296,6 +296,22 @@ MECHANISMS = {
         [parallel(mlp=moe_ff(experts=5, top=1, ff=8, limit=0.3, shared=8,
                              shared_limit=0.2))], 2, True),
     "one-stream-plain-residual": ([parallel(mlp=moe_ff())], 1, False),
+    # head and latent sizes that the bf16 MFMA prefill and split-KV
+    # decode kernels serve (64 and 128), the latent cache as key AND
+    # value operand of those kernels
+    "parallel-d64-tiles": (
+        [parallel(heads=4, kv_heads=2, dim=64, vdim=64, rot_dims=16,
+                  window=11, scale=0.1)], 2, True),
+    "parallel-d128-tiles": (
+        [parallel(heads=2, kv_heads=1, dim=128, vdim=128, rot_dims=128,
+                  window=40, scale=0.07, softcap=3.0)], 2, True),
+    "latent-rank64-tiles": (
+        [latent(heads=4, dim=16, vdim=8, kv_rank=64, q_rank=24),
+         latent(heads=2, dim=8, vdim=24, kv_rank=64, q_rank=8,
+                kv_from=0)], 2, True),
+    "latent-rank128-tiles": (
+        [latent(heads=4, dim=32, vdim=16, kv_rank=128, q_rank=40,
+                scale=0.2)], 3, True),
 }
 
 
@@ -312,8 +328,11 @@ def test_each_mechanism_alone(name, device, dtype, width):
     w = make_weights(cfg, 1, hc=hc)
     llm = engine(save_model(cfg, w), device, dtype)
     toks = tokens_for(cfg, 37, 2)
-    got = run_steps(llm, cut("a", toks, [37]), cfg["vocab"])
-    check_against_oracle(cfg, w, got, {"a": toks}, TOL[dtype])
+    # the whole prompt, then the same prompt as a portion and decoding
+    # (a second request: other pages, the decode kernels)
+    steps = cut("a", toks, [37]) + cut("b", toks, [30] + [1] * 7)
+    got = run_steps(llm, steps, cfg["vocab"])
+    check_against_oracle(cfg, w, got, {"a": toks, "b": toks}, TOL[dtype])
 
 
 @pytest.mark.parametrize("device,dtype", DEVICES)
