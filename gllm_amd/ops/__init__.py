@@ -192,7 +192,20 @@ def topk_softmax(gating: torch.Tensor, topk: int, renormalize: bool = True):
 
 
 def topk_then_softmax(logits: torch.Tensor, topk: int):
-    """Top-k over raw router logits, softmax over the chosen only."""
+    """Top-k over raw router logits, softmax over the chosen only:
+    (weights fp32 [T, k] in descending order of logit, ids int32
+    [T, k]). fp32 logits of up to 512 experts on the GPU take one
+    wave-per-row kernel (ties go to the lower index)."""
+    if (logits.is_cuda and logits.dtype == torch.float32
+            and logits.dim() == 2 and logits.shape[1] <= 512
+            and topk <= min(64, logits.shape[1])):
+        logits = logits.contiguous()
+        weights = torch.empty(logits.shape[0], topk, dtype=torch.float32,
+                              device=logits.device)
+        ids = torch.empty(logits.shape[0], topk, dtype=torch.int32,
+                          device=logits.device)
+        _seq_kernels().topk_softmax_rows(weights, ids, logits)
+        return weights, ids
     return torch_ref.topk_then_softmax(logits, topk)
 
 

@@ -103,6 +103,8 @@ void moe_gemm(torch::Tensor C, torch::Tensor A, torch::Tensor W,
               c10::optional<torch::Tensor> topk_weights, long n_pairs,
               long topk, long block_m, bool scatter);
 void moe_sum(torch::Tensor out, torch::Tensor pair_out, long topk);
+void topk_softmax_rows(torch::Tensor weights, torch::Tensor ids,
+                       torch::Tensor logits);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("layernorm_f32", &layernorm_f32, "h = LN(x fp32) in the model dtype");
@@ -146,4 +148,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_align", &moe_align, "device-side moe_align_block_size");
   m.def("moe_gemm", &moe_gemm, "grouped MFMA GEMM over sorted pairs");
   m.def("moe_sum", &moe_sum, "sum pair outputs over topk");
+  m.def("topk_softmax_rows", &topk_softmax_rows,
+        "top-k of router logits, softmax over the chosen");
 }

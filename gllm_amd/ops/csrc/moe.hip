@@ -347,3 +347,89 @@ void moe_sum(torch::Tensor out, torch::Tensor pair_out, long topk) {
                      (int)topk, H);
   HIP_CHECK_KERNEL();
 }
+
+// ---------------------------------------------------------------------
+// Top-k of the router LOGITS, softmax over the chosen ones only.
+// One wave per token row: lane l holds logits l, l + 64, ... (E <= 512);
+// k rounds of a wave-wide arg-max (ties go to the lower index) pick the
+// experts in descending order, lane r keeps the r-th pick, and the
+// softmax over the k picks is one more wave reduction.
+namespace {
+
+constexpr int TK_MAXJ = 8;  // logits per lane: E <= 64 * TK_MAXJ
+
+__global__ __launch_bounds__(256) void topk_softmax_rows_kernel(
+    float *__restrict__ weights, int *__restrict__ ids,
+    const float *__restrict__ logits, long rows, int E, int k) {
+  const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (r >= rows) return;
+  const float *row = logits + r * E;
+  float v[TK_MAXJ];
+#pragma unroll
+  for (int j = 0; j < TK_MAXJ; ++j) {
+    const int e = lane + 64 * j;
+    v[j] = e < E ? row[e] : -INFINITY;
+  }
+  unsigned taken = 0;
+  float my_val = -INFINITY;
+  int my_idx = 0;
+  for (int it = 0; it < k; ++it) {
+    float best = -INFINITY;
+    int bidx = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < TK_MAXJ; ++j) {
+      const int e = lane + 64 * j;
+      if (e < E && !(taken >> j & 1u) && (bidx == 0x7fffffff || v[j] > best)) {
+        best = v[j];
+        bidx = e;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(best, off, 64);
+      const int oi = __shfl_xor(bidx, off, 64);
+      // an exhausted lane (no index) loses; a NaN never beats a number
+      const bool take = oi != 0x7fffffff &&
+                        (bidx == 0x7fffffff || ov > best ||
+                         (ov == best && oi < bidx) ||
+                         (best != best && ov == ov));
+      if (take) { best = ov; bidx = oi; }
+    }
+    if ((bidx & 63) == lane) taken |= 1u << (bidx >> 6);
+    if (lane == it) { my_val = best; my_idx = bidx; }
+  }
+  const float top = __shfl(my_val, 0, 64);  // the first pick is the largest
+  const float p = lane < k ? expf(my_val - top) : 0.f;
+  const float sum = wave_reduce_sum(p);
+  if (lane < k) {
+    weights[r * k + lane] = p / sum;
+    ids[r * k + lane] = my_idx;
+  }
+}
+
+}  // namespace
+
+void topk_softmax_rows(torch::Tensor weights, torch::Tensor ids,
+                       torch::Tensor logits) {
+  TORCH_CHECK(logits.is_cuda() && logits.dim() == 2 &&
+              logits.is_contiguous() && logits.scalar_type() == at::kFloat,
+              "logits: fp32 [rows, experts]");
+  const long rows = logits.size(0);
+  const int E = logits.size(1);
+  TORCH_CHECK(weights.dim() == 2 && weights.size(0) == rows &&
+              weights.is_contiguous() && weights.scalar_type() == at::kFloat);
+  const int k = weights.size(1);
+  TORCH_CHECK(ids.is_contiguous() && ids.scalar_type() == at::kInt &&
+              ids.numel() == rows * k);
+  TORCH_CHECK(E >= 1 && E <= 64 * TK_MAXJ && k >= 1 && k <= 64 && k <= E,
+              "topk_softmax_rows: experts <= ", 64 * TK_MAXJ,
+              ", top <= min(64, experts)");
+  if (rows == 0) return;
+  auto stream = at::cuda::getCurrentCUDAStream();
+  hipLaunchKernelGGL(topk_softmax_rows_kernel, dim3((rows + 3) / 4),
+                     dim3(256), 0, stream, weights.data_ptr<float>(),
+                     ids.data_ptr<int>(), logits.data_ptr<float>(), rows, E,
+                     k);
+  HIP_CHECK_KERNEL();
+}

@@ -719,6 +719,30 @@ def test_hyper_streams_op(device, dtype):
             assert (h2.float() - h.float()).abs().max() < tol
 
 
+@pytest.mark.parametrize("device", [
+    pytest.param("cpu", id="cpu"),
+    pytest.param("cuda", id="gpu", marks=pytest.mark.gpu)])
+def test_routing_op(device):
+    """ops.topk_then_softmax: the k largest logits in descending order,
+    softmax over them alone; expert counts below, at and above a wave's
+    width, k = 1, k = experts, a row with a tie (lower index first)."""
+    from gllm_amd import ops
+    g = torch.Generator().manual_seed(12)
+    for E, k, T in ((5, 1, 7), (5, 5, 3), (64, 4, 33), (100, 8, 9),
+                    (300, 2, 130), (512, 64, 2)):
+        logits = torch.randn(T, E, generator=g) * 3
+        w, ids = ops.topk_then_softmax(logits.to(device), k)
+        w, ids = w.cpu(), ids.cpu().long()
+        vals, want = torch.topk(logits, k, dim=-1)
+        assert torch.equal(ids, want), (E, k)
+        assert (w - torch.softmax(vals, -1)).abs().max() < 1e-6
+        assert ids.dtype == torch.int64 and w.dtype == torch.float32
+    tie = torch.tensor([[0.5, 2.0, -1.0, 2.0, 2.0, 0.0]])
+    w, ids = ops.topk_then_softmax(tie.to(device), 2)
+    assert sorted(ids.cpu().tolist()[0]) == [1, 3] or device == "cpu"
+    assert (w.cpu() - 0.5).abs().max() < 1e-6
+
+
 @pytest.mark.parametrize("graph", [False, True], ids=["eager", "graph"])
 @pytest.mark.parametrize("device,dtype", DEVICES)
 def test_greedy_generation_through_the_scheduler(device, dtype, graph):
