@@ -297,10 +297,10 @@ def gopetar_config(sz, vocab=32000, window=4096, streams=2):
                 "left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D,
                          "scale": D ** -0.5, "softcap": 30.0,
                          "mask": {"size": window},
-                         "rot": {"dims": D // 2, "base": 500000.0,
-                                 "scaling": {"factor": 8.0, "low": 1.0,
-                                             "high": 4.0,
-                                             "original": 8192}}},
+                         "rot": {"dims": D // 2, "base": 1000000.0,
+                                 "scaling": {"factor": 4.0, "low": 1.0,
+                                             "high": 8.0,
+                                             "original": 4096}}},
                 "left_scale": 0.5, "right": {"width": sz["width"]},
                 "right_scale": 0.5}})
     return {"architecture": "Gopetar", "embedding": {"scale": 1.0},
