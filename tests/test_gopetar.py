@@ -781,6 +781,42 @@ def test_greedy_generation_through_the_scheduler(device, dtype, graph):
     assert checked >= 8
 
 
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_prefix_cache_hit_restores_state(device, dtype):
+    """A second prompt that shares two full pages with an earlier one
+    re-uses the cached K/V and latent pages and the minGRU state
+    snapshot taken at that page boundary; its greedy continuation still
+    matches the oracle."""
+    from gllm_amd.config import EngineConfig
+    from gllm_amd.engine.llm import LLM
+    from gllm_amd.sequence import SamplingParams
+    cfg = make_config(stack_for(dtype), width=32, vocab=48, streams=2)
+    w = make_weights(cfg, 21)
+    config = EngineConfig(model=save_model(cfg, w), dtype=dtype,
+                          device=device, page_size=16, maxp=16, maxd=8,
+                          use_graph=False, enable_overlap=False,
+                          enable_prefix_caching=True)
+    llm = LLM(config=config, num_pages_override=64)
+    first = tokens_for(cfg, 48, 31)
+    second = first[:32] + tokens_for(cfg, 9, 32)
+    sp = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    llm.generate([first], sp)
+    hit_before = llm.runner.memory_manager.hit_tokens
+    out = llm.generate([second], sp)[0]
+    assert llm.runner.memory_manager.hit_tokens - hit_before == 32
+    margin = 0.05 if dtype == "float32" else 0.5
+    seq, checked = list(second), 0
+    for tok in out.token_ids:
+        logits = oracle.forward(cfg, w, seq)[-1]
+        top2 = torch.topk(logits, 2).values
+        if float(top2[0] - top2[1]) >= margin:
+            assert tok == int(logits.argmax()), (len(seq), tok)
+            checked += 1
+        seq.append(tok)
+    # (bf16 needs a wide margin to call a token decided; few qualify)
+    assert checked >= (3 if dtype == "float32" else 1)
+
+
 def test_config_and_registry():
     """The loader picks the class from config.json's architecture key;
     a parallel layer owns a K/V cache and a state entry, a latent layer
