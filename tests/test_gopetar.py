@@ -61,9 +61,10 @@ def latent(heads=3, dim=8, vdim=10, kv_rank=12, q_rank=14, scale=0.4,
     return {"type": "latent_attention", "mixer": m, "mlp": mlp}
 
 
-# wavelengths 2 pi / f of base 100 over 8 dims: 6.3, 20, 63, 199 — one
-# pair on each side of the blend and two inside it
-SCALING = {"factor": 4.0, "low": 1.0, "high": 8.0, "original": 96}
+# wavelengths 2 pi / f of base 100 over 8 dims: 6.3, 20, 63, 199; with
+# original/high = 12 and original/low = 48 the first pair keeps its
+# frequency, the second is blended, the last two are slowed
+SCALING = {"factor": 4.0, "low": 2.0, "high": 8.0, "original": 96}
 
 
 def make_config(layers, width=32, vocab=70, eps=1e-5, streams=2,
