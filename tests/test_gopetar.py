@@ -779,7 +779,8 @@ def test_greedy_generation_through_the_scheduler(device, dtype, graph):
                 assert tok == int(logits.argmax()), (len(seq), tok)
                 checked += 1
             seq.append(tok)
-    assert checked >= 8
+    # (bf16 needs a wide margin to call a token decided; fewer qualify)
+    assert checked >= (8 if dtype == "float32" else 3)
 
 
 @pytest.mark.parametrize("device,dtype", DEVICES)
