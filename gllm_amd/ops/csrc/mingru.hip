@@ -19,6 +19,8 @@
 // earlier segments applied to the carried state give the segment's
 // start state; pass 2 replays the segment from there and writes the
 // outputs. A decode-only batch runs NSEG = 1 (one pass, nothing folded).
+// CH x NSEG is 64 x 16, or 32 x 32 / 16 x 64 for small batches, so that a
+// few long sequences still give every compute unit a workgroup.
 
 #include <torch/extension.h>
 #include <ATen/cuda/CUDAContext.h>
@@ -123,9 +125,16 @@ void mingru_varlen(torch::Tensor out, torch::Tensor zx, torch::Tensor gp,
                      state.data_ptr<float>(), slots.data_ptr<long>(),       \
                      has_init.data_ptr<int>(),                              \
                      query_start_loc.data_ptr<int>(), C, (float)scale)
+  // batches with prompt portions: 1024 threads = CH channels x NSEG
+  // segments; fewer channels per workgroup (more, shorter segments) when
+  // 64 would leave compute units without a workgroup
+  const long wg64 = (long)B * ((C + 63) / 64);
+  const int ch = wg64 >= 256 ? 64 : (2 * wg64 >= 256 ? 32 : 16);
 #define RUN_T(TT)                                                           \
   if (max_query_len > 0 && max_query_len <= 8) RUN(TT, 256, 1);             \
-  else RUN(TT, 64, 16)
+  else if (ch == 64) RUN(TT, 64, 16);                                       \
+  else if (ch == 32) RUN(TT, 32, 32);                                       \
+  else RUN(TT, 16, 64)
   if (st == at::kBFloat16) { RUN_T(__hip_bfloat16); }
   else if (st == at::kFloat) { RUN_T(float); }
   else TORCH_CHECK(false, "mingru_varlen: bf16 or fp32");

@@ -666,6 +666,30 @@ def test_mingru_state_carries_and_restarts(device, dtype):
     tol = 1e-5 if dtype == "float32" else 3e-2
     assert (out.double() - want).abs().max() < tol
     assert (st.cpu().double() - final).abs().max() < 1e-5
+    # many sequences x many channels: the wider workgroup shapes
+    for B, C2 in ((40, 512), (20, 512)):
+        lens2 = [9 + (7 * b) % 50 for b in range(B)]
+        T2 = sum(lens2)
+        zx2 = torch.randn(T2, 2 * C2, generator=g).to(tdt)
+        gp2 = torch.randn(T2, C2, generator=g).to(tdt)
+        st2 = torch.zeros(B + 1, C2, device=device)
+        qsl2 = torch.tensor([0] + list(np.cumsum(lens2)), dtype=torch.int32)
+        o2 = ops.mingru_varlen(
+            zx2.to(device), gp2.to(device), st2,
+            torch.arange(B).to(device),
+            torch.zeros(B, dtype=torch.int32, device=device),
+            qsl2.to(device), 1.0, max(lens2)).float().cpu().double()
+        z2 = torch.sigmoid(zx2[:, :C2].double())
+        u2 = zx2[:, C2:].double()
+        c2 = torch.where(u2 >= 0, u2 + 0.5, torch.sigmoid(u2))
+        g2 = gp2.double()
+        for b in (0, B // 2, B - 1):
+            S = torch.zeros(C2, dtype=torch.float64)
+            for t in range(int(qsl2[b]), int(qsl2[b + 1])):
+                S = (1 - z2[t]) * S + z2[t] * c2[t]
+                assert (o2[t] - S * g2[t] * torch.sigmoid(g2[t])
+                        ).abs().max() < tol, (B, b, t)
+            assert (st2[b].cpu().double() - S).abs().max() < 1e-5
     # decode-only batch over the same slots
     zx1, gp1 = zx[:5].to(device), gp[:5].to(device)
     st2 = st.clone()
