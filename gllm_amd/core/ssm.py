@@ -49,6 +49,9 @@ class SSMLayerSpec:
     # itself (an element-wise gated recurrence: (channels,)); conv_dim 0
     # = the layer has no short convolution and holds no conv state
     state_shape: Optional[tuple] = None
+    # token shift: the layer also keeps the last row its mixer read
+    # ([slots, shift_dim] in the pool's dtype); 0 = none
+    shift_dim: int = 0
 
 
 class SSMPool:
@@ -70,6 +73,9 @@ class SSMPool:
                     (ls.head_k_dim, ls.head_v_dim) if ls.layout == "kv"
                     else (ls.head_v_dim, ls.head_k_dim)),
                 dtype=torch.float32, device=device) for ls in spec.layers]
+            self.shift_state = [torch.zeros(
+                num_slots, ls.shift_dim, dtype=dtype, device=device)
+                for ls in spec.layers]
         else:
             self.conv_state = torch.zeros(
                 L, num_slots, spec.conv_dim, spec.conv_kernel - 1,
@@ -113,7 +119,8 @@ class SSMPool:
         snaps = self.snapshots
         if isinstance(self.conv_state, list):
             snaps[chain_id] = ([c[slot].clone() for c in self.conv_state],
-                               [r[slot].clone() for r in self.ssm_state])
+                               [r[slot].clone() for r in self.ssm_state],
+                               [m[slot].clone() for m in self.shift_state])
         else:
             snaps[chain_id] = (self.conv_state[:, slot].clone(),
                                self.ssm_state[:, slot].clone())
@@ -131,6 +138,8 @@ class SSMPool:
                 c[slot].copy_(sc)
             for r, sr in zip(self.ssm_state, snap[1]):
                 r[slot].copy_(sr)
+            for m, sm in zip(self.shift_state, snap[2]):
+                m[slot].copy_(sm)
         else:
             self.conv_state[:, slot].copy_(snap[0])
             self.ssm_state[:, slot].copy_(snap[1])

@@ -68,6 +68,11 @@ class WindowAttention(nn.Module):
       value of position j enters the cache turned by j, and each head's
       weighted sum at position i is turned back by i, so what a query
       receives from a key depends on their distance only
+    * ``norm_span``: q (and k) get ONE RMS over all heads of the token
+      with weights that cover the whole row ([H*D], [G*D]) instead of a
+      norm per head; ``value_unit_norm``: every value head enters the
+      cache divided by its RMS (eps, no weight). A ``rotary`` with
+      ``half_layout`` pairs dimension i with i + rot_dims/2
     * ``kv_source``: cache index of ANOTHER layer whose keys and values
       this layer attends over; such a layer owns no k/v tensors and
       stores nothing (``owns_kv`` False)
@@ -81,9 +86,12 @@ class WindowAttention(nn.Module):
                  rotary: Optional[nn.Module] = None, owns_kv: bool = True,
                  params_dtype=None, qk_norm: bool = True,
                  softcap: float = 0.0,
-                 value_rotary: Optional[nn.Module] = None):
+                 value_rotary: Optional[nn.Module] = None,
+                 norm_span: bool = False, value_unit_norm: bool = False):
         super().__init__()
         dtype = params_dtype or torch.get_default_dtype()
+        self.norm_span = norm_span
+        self.value_unit_norm = value_unit_norm
         self.layer_idx = layer_idx       # cache this layer reads
         self.num_heads = num_heads
         self.num_kv_heads = num_kv_heads
@@ -102,11 +110,13 @@ class WindowAttention(nn.Module):
         if value_rotary is not None:
             assert value_rotary.rot_dims == v_head_dim
         if qk_norm:
-            self.q_norm = nn.Parameter(torch.ones(head_dim, dtype=dtype),
+            nq = num_heads * head_dim if norm_span else head_dim
+            nk = num_kv_heads * head_dim if norm_span else head_dim
+            self.q_norm = nn.Parameter(torch.ones(nq, dtype=dtype),
                                        requires_grad=False)
             if owns_kv:
                 self.k_norm = nn.Parameter(
-                    torch.ones(head_dim, dtype=dtype), requires_grad=False)
+                    torch.ones(nk, dtype=dtype), requires_grad=False)
         else:
             self.q_norm = self.k_norm = None
         if sink == "learned":
@@ -127,20 +137,25 @@ class WindowAttention(nn.Module):
     def forward(self, q: torch.Tensor, k: Optional[torch.Tensor],
                 v: Optional[torch.Tensor], gate: Optional[torch.Tensor],
                 fctx: ForwardContext, out: Optional[torch.Tensor] = None,
-                out_scale: float = 1.0) -> torch.Tensor:
+                out_scale: float = 1.0,
+                layer_idx: Optional[int] = None) -> torch.Tensor:
         """q [T, H*D], k [T, G*D], v [T, G*Dv], gate [T, H*Dv] (row
         views of a merged projection are fine). Returns [T, H*Dv],
         multiplied by ``out_scale`` and written into ``out`` (which may
-        be a column block of a wider buffer) when those are given."""
+        be a column block of a wider buffer) when those are given.
+        ``layer_idx`` overrides the cache index (a layer that runs
+        several times keeps one cache per run)."""
         T = q.shape[0]
+        idx = self.layer_idx if layer_idx is None else layer_idx
         if fctx.is_profile_run:
             if out is not None:
                 out.zero_()
                 return out
             return q.new_zeros(T, self.num_heads * self.v_head_dim)
-        k_cache = fctx.k_caches[self.layer_idx]
-        v_cache = fctx.v_caches[self.layer_idx]
+        k_cache = fctx.k_caches[idx]
+        v_cache = fctx.v_caches[idx]
         freqs, mag, rot_dims = self._freqs(q.device)
+        half = bool(getattr(self.rotary, "half_layout", False))
         vrot = self.value_rotary
         vfreqs = vrot.freqs if vrot is not None else None
         if self.owns_kv:
@@ -148,14 +163,16 @@ class WindowAttention(nn.Module):
                 q, k, v, self.q_norm, self.k_norm, fctx.positions,
                 fctx.slot_mapping, freqs, mag, rot_dims, k_cache, v_cache,
                 self.num_heads, self.num_kv_heads, self.head_dim,
-                self.v_head_dim, self.eps, do_norm=self.qk_norm,
-                v_freqs=vfreqs)
+                self.v_head_dim, self.eps, half_layout=half,
+                do_norm=self.qk_norm, v_freqs=vfreqs,
+                norm_span=self.norm_span, v_unit=self.value_unit_norm)
         else:
             ops.qk_norm_rope_store(
                 q, None, None, self.q_norm, None, fctx.positions,
                 fctx.slot_mapping, freqs, mag, rot_dims, None, None,
                 self.num_heads, self.num_kv_heads, self.head_dim,
-                self.v_head_dim, self.eps, do_norm=self.qk_norm)
+                self.v_head_dim, self.eps, half_layout=half,
+                do_norm=self.qk_norm, norm_span=self.norm_span)
         o = ops.window_attention(
             q, gate, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
             fctx.query_start_loc, self.scale, self.window,

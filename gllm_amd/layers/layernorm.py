@@ -100,3 +100,40 @@ class LayerNorm(nn.Module):
         pre = (nxt.weight, nxt.bias) if nxt is not None else None
         return ops.residual_layernorm(x, y, self.weight, self.bias,
                                       self.eps, pre, gate)
+
+
+class StreamRMSNorm(nn.Module):
+    """RMS norm (plain weight, eps inside the root) over an fp32
+    residual stream, for decoders that norm before AND after every
+    sublayer and add the normed result times a fixed multiplier:
+
+    * ``norm(x)``                          h = RMSnorm(x) * w, model dtype
+    * ``norm.add_into(x, y, nxt, mult)``   x += mult * RMSnorm(y) * w in
+      place and, with ``nxt`` (the next sublayer's pre-norm), returns
+      nxt(x): one launch per boundary (ops.stream_rmsnorm)
+    * ``y2``: the norm sees y + y2 (a routed and a shared result);
+      ``y_scale``: it sees y_scale * (y + y2), the product formed in
+      fp32; ``add`` (fp32 [width]): added to every row of x after the
+      sublayer result and before ``nxt`` reads it
+    """
+
+    def __init__(self, hidden_size: int, eps: float = 1e-5,
+                 params_dtype=None):
+        super().__init__()
+        dtype = params_dtype or torch.get_default_dtype()
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype),
+                                   requires_grad=False)
+        self.eps = eps
+
+    def forward(self, x: torch.Tensor,
+                add: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.stream_rmsnorm(x, None, None, self.eps, add=add,
+                                  pre_w=self.weight)
+
+    def add_into(self, x: torch.Tensor, y: torch.Tensor,
+                 nxt: Optional["StreamRMSNorm"] = None, mult: float = 1.0,
+                 y_scale: float = 1.0, y2: Optional[torch.Tensor] = None,
+                 add: Optional[torch.Tensor] = None):
+        return ops.stream_rmsnorm(
+            x, y, self.weight, self.eps, mult, y_scale, y2, add,
+            nxt.weight if nxt is not None else None)

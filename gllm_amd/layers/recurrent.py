@@ -1,7 +1,8 @@
-"""Element-wise gated recurrences served from the per-sequence state
-pool (core/ssm.py)."""
+"""Recurrent mixers and token shift served from the per-sequence
+state pool (core/ssm.py)."""
 
-from typing import List
+import math
+from typing import List, Optional
 
 import torch
 import torch.nn as nn
@@ -80,3 +81,101 @@ class MinGRU(nn.Module):
         return ops.mingru_varlen(
             zx, gp, fctx.ssm_pool.ssm_state[self.ssm_layer_id], slots, init,
             fctx.query_start_loc, scale, fctx.max_query_len, out)
+
+
+_ONES = {}
+
+
+def state_rows(fctx: ForwardContext, T: int, device):
+    """(slots, carried-state flags) of a batch for the ragged state
+    kernels. Inside a captured decode bucket every row is a one-token
+    step on carried state and the slots come from the runner's
+    persistent buffer (padding rows work on the pool's scratch slot)."""
+    if fctx.ssm_slots_dev is not None:
+        ones = _ONES.get(device)
+        if ones is None or ones.numel() < T:
+            ones = _ONES[device] = torch.ones(
+                max(T, 1024), dtype=torch.int32, device=device)
+        return fctx.ssm_slots_dev[:T], ones[:T]
+    return fctx.ssm_slots_t, fctx.ssm_has_init_t
+
+
+class TokenShift(nn.Module):
+    """h_t <- h_t + (h_(t-1) - h_t) * mu, per channel, h_(t-1) being the
+    previous token's row as it came in (zeros ahead of a sequence's
+    first token). The last incoming row of every sequence lives in the
+    state pool (``shift_state[ssm_layer_id]``), so prompt portions and
+    decode steps continue each other."""
+
+    def __init__(self, width: int, ssm_layer_id: int, params_dtype=None):
+        super().__init__()
+        dtype = params_dtype or torch.get_default_dtype()
+        self.ssm_layer_id = ssm_layer_id
+        self.mu = nn.Parameter(torch.zeros(width, dtype=dtype),
+                               requires_grad=False)
+
+    def forward(self, h: torch.Tensor, fctx: ForwardContext,
+                ssm_layer_id: Optional[int] = None) -> torch.Tensor:
+        if fctx.is_profile_run or fctx.ssm_pool is None:
+            return h
+        sid = self.ssm_layer_id if ssm_layer_id is None else ssm_layer_id
+        slots, init = state_rows(fctx, h.shape[0], h.device)
+        return ops.token_shift(h, self.mu, fctx.ssm_pool.shift_state[sid],
+                               slots, init, fctx.query_start_loc)
+
+
+class GeneralDeltaRule(nn.Module):
+    """Delta rule with a decay per key channel and a removal rate per
+    key channel, ``heads`` heads of key size ``dim`` and value size
+    ``vdim``:
+
+        w_t = exp(-decay_scale * sigmoid(w_logit_t + w0))
+        a_t = sigmoid(a_logit_t)       u_t = k_t / sqrt(|k_t|^2 + 1e-6)
+        S_t = diag(w_t) S_(t-1) - (a_t u_t)(u_t^T S_(t-1)) + k_t v_t^T
+        o_t = S_t^T r_t
+
+    and a read-out scale * o / rms(o) * norm_weight * sigmoid(gate) per
+    head (``norm_weight`` [heads * vdim]: every head has its own). The
+    caller owns the projections (r, k, v, the two logit rows, the gate;
+    row views of a merged projection are fine); decay, removal rate,
+    unit key and the state [slots, heads, dim, vdim] are fp32.
+    """
+
+    def __init__(self, heads: int, dim: int, vdim: int, eps: float,
+                 ssm_layer_id: int, decay_scale: float = math.exp(-0.5),
+                 params_dtype=None):
+        super().__init__()
+        dtype = params_dtype or torch.get_default_dtype()
+        self.heads, self.dim, self.vdim = heads, dim, vdim
+        self.eps = eps
+        self.decay_scale = float(decay_scale)
+        self.ssm_layer_id = ssm_layer_id
+        self.w0 = nn.Parameter(torch.zeros(heads * dim, dtype=dtype),
+                               requires_grad=False)
+        self.norm_weight = nn.Parameter(
+            torch.ones(heads * vdim, dtype=dtype), requires_grad=False)
+
+    def spec(self, conv_dim: int = 0, conv_kernel: int = 1,
+             shift_dim: int = 0) -> SSMLayerSpec:
+        """Pool geometry of one run of the layer; a sibling's short
+        convolution and a token shift ride on the same entry."""
+        return SSMLayerSpec(conv_dim, conv_kernel, self.heads, self.dim,
+                            self.vdim, layout="kv", shift_dim=shift_dim)
+
+    def forward(self, r, k, v, w_logit, a_logit, gate,
+                fctx: ForwardContext, out: torch.Tensor = None,
+                scale: float = 1.0, ssm_layer_id: Optional[int] = None):
+        T = r.shape[0]
+        if fctx.is_profile_run or fctx.ssm_pool is None:
+            if out is not None:
+                out.zero_()
+                return out
+            return r.new_zeros(T, self.heads * self.vdim)
+        sid = self.ssm_layer_id if ssm_layer_id is None else ssm_layer_id
+        slots, init = state_rows(fctx, T, r.device)
+        o = ops.general_delta_rule(
+            r, k, v, w_logit, a_logit, self.w0, self.decay_scale,
+            fctx.ssm_pool.ssm_state[sid], slots, init,
+            fctx.query_start_loc, fctx.max_query_len)
+        return ops.rms_gate(o, gate, self.norm_weight, self.heads, self.eps,
+                            r.dtype, gate="sigmoid", scale=scale, out=out)

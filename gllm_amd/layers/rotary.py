@@ -260,16 +260,25 @@ class HalfRotary(nn.Module):
     Like PairRotary it holds only the fp64 per-pair frequencies; the
     fused q/k kernel (ops.qk_norm_rope_store with ``half_layout``) forms
     position * frequency in fp64, so no position table is sized.
+
+    ``scaling`` = dict(factor): linear position scaling, every
+    frequency divided by ``factor``.
     """
 
     half_layout = True
     mag = 1.0
 
-    def __init__(self, rot_dims: int, base: float):
+    def __init__(self, rot_dims: int, base: float,
+                 scaling: Optional[dict] = None):
         super().__init__()
         assert rot_dims % 2 == 0
         self.rot_dims = rot_dims
         i = torch.arange(rot_dims // 2, dtype=torch.float64)
         freqs = torch.pow(torch.tensor(float(base), dtype=torch.float64),
                           -2.0 * i / max(rot_dims, 1))
+        if scaling:
+            extra = set(scaling) - {"factor"}
+            if extra:
+                raise ValueError(f"unknown rotary scaling keys {extra}")
+            freqs = freqs / float(scaling.get("factor", 1.0))
         self.register_buffer("freqs", freqs, persistent=False)

@@ -36,7 +36,9 @@ def get_arch_registry():
     from gllm_amd.models.sudevik import SudevikForCausalLM
     from gllm_amd.models.gukirax import GukiraxForCausalLM
     from gllm_amd.models.gopetar import GopetarForCausalLM
+    from gllm_amd.models.sofunex import SofunexForCausalLM
     return {
+        "Sofunex": SofunexForCausalLM,
         "Gopetar": GopetarForCausalLM,
         "Sudevik": SudevikForCausalLM,
         "Gukirax": GukiraxForCausalLM,

@@ -791,11 +791,62 @@ def residual_layernorm(x: torch.Tensor, y: torch.Tensor, w_post, b_post,
                                         gate)
 
 
+def stream_rmsnorm(x: torch.Tensor, y, w_post, eps: float,
+                   mult: float = 1.0, y_scale: float = 1.0, y2=None,
+                   add=None, pre_w=None):
+    """One launch per sublayer boundary of an RMS sandwich-norm decoder
+    over an fp32 stream x (in place):
+        x += mult * RMSnorm(y_scale * (y + y2)) * w_post   (y given)
+        x += add                                           (add: fp32 [width])
+        returns RMSnorm(x) * pre_w in pre_w's dtype        (pre_w given)
+    y / y2 may be row views; statistics and sums are fp32."""
+    if x.is_cuda:
+        h = None
+        if pre_w is not None:
+            h = torch.empty(x.shape, dtype=pre_w.dtype, device=x.device)
+        _seq_kernels().stream_rmsnorm(x, y, y2, w_post, add, h, pre_w,
+                                      float(eps), float(mult),
+                                      float(y_scale))
+        return h
+    return torch_ref.stream_rmsnorm(x, y, w_post, eps, mult, y_scale, y2,
+                                    add, pre_w)
+
+
+def gelu_tanh_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """x [rows, 2d] = gate | up -> gelu_tanh(gate) * up."""
+    if x.is_cuda:
+        d = x.shape[-1] // 2
+        out = torch.empty(x.shape[:-1] + (d,), dtype=x.dtype,
+                          device=x.device)
+        _seq_kernels().gelu_tanh_and_mul(out, x)
+        return out
+    return torch_ref.gelu_tanh_and_mul(x)
+
+
+def sigmoid_group_topk(logits: torch.Tensor, correction, topk: int,
+                       n_group: int = 1, keep: int = 1,
+                       scale: float = 1.0):
+    """Sigmoid router with a selection-only correction and group
+    limits, one kernel on the GPU. logits fp32 [T, E]; returns (weights
+    fp32 [T, topk], ids int32 [T, topk]). See torch_ref for the rule."""
+    if logits.is_cuda:
+        T = logits.shape[0]
+        weights = torch.empty(T, topk, dtype=torch.float32,
+                              device=logits.device)
+        ids = torch.empty(T, topk, dtype=torch.int32, device=logits.device)
+        _seq_kernels().sigmoid_group_topk(weights, ids, logits, correction,
+                                          int(n_group), int(keep),
+                                          float(scale))
+        return weights, ids
+    return torch_ref.sigmoid_group_topk(logits, correction, topk, n_group,
+                                        keep, scale)
+
+
 # --------------------------------------------------------------- windowed attn
 def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
                        mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
                        half_layout=False, norm_last=False, do_norm=True,
-                       v_freqs=None):
+                       v_freqs=None, norm_span=False, v_unit=False):
     """Fused per-head q/k RMS norm, rotary (per-pair frequency table
     ``freqs`` fp64, cos/sin scaled by ``mag``) and paged K/V store.
     q [T, H*D] is updated in place (may be a column slice of a merged
@@ -807,17 +858,23 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
     ``v`` may be ``k`` itself (values = keys as projected).
     ``do_norm`` False: rotary and store only. ``v_freqs`` (fp64
     [Dv/2]): each value row is turned by its own position over all of
-    Dv (same pair layout) on its way into the cache."""
+    Dv (same pair layout) on its way into the cache.
+    ``norm_span``: one RMS over all heads of a token's q (and of its k)
+    with weights that cover the row ([H*D], [G*D]). ``v_unit``: each
+    value head is divided by its RMS (eps inside the root, no weight)
+    before it is stored."""
     if q.is_cuda:
         _seq_kernels().qk_norm_rope_store(
             q, k, v, q_w, k_w, positions, slot_mapping, freqs, mag,
             rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
-            bool(half_layout), bool(norm_last), bool(do_norm), v_freqs)
+            bool(half_layout), bool(norm_last), bool(do_norm), v_freqs,
+            bool(norm_span), bool(v_unit))
         return
     torch_ref.qk_norm_rope_store(q, k, v, q_w, k_w, positions,
                                  slot_mapping, freqs, mag, rot_dims,
                                  k_cache, v_cache, H, G, D, Dv, eps,
-                                 half_layout, norm_last, do_norm, v_freqs)
+                                 half_layout, norm_last, do_norm, v_freqs,
+                                 norm_span, v_unit)
 
 
 def rotate_scale_rows(x, positions, freqs, heads, D, sign=1.0, scale=1.0,
@@ -999,17 +1056,20 @@ def relu2(x: torch.Tensor) -> torch.Tensor:
 
 
 # --------------------------------------------------------------- delta rule
-def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc):
-    """Ragged short causal conv + silu; rolls ``conv_state`` rows
-    ``slots`` in place. x may be a column slice of a merged projection."""
+def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc,
+                     activation=True):
+    """Ragged short causal conv + silu (``activation`` False: the plain
+    convolution); rolls ``conv_state`` rows ``slots`` in place. x may be
+    a column slice of a merged projection."""
     if x.is_cuda:
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         _seq_kernels().causal_conv_silu(out, x, w, conv_state, slots,
-                                        has_init, query_start_loc)
+                                        has_init, query_start_loc,
+                                        bool(activation))
         return out
     from gllm_amd.ops import gdn_ref
     return gdn_ref.causal_conv_silu(x, w, conv_state, slots, has_init,
-                                    query_start_loc)
+                                    query_start_loc, activation)
 
 
 def delta_rule_varlen(q, k, v, a, b, A_log, dt_bias, state, slots,
@@ -1035,12 +1095,58 @@ def delta_rule_varlen(q, k, v, a, b, A_log, dt_bias, state, slots,
                                      q_scale)
 
 
-def rms_gate(o, z, w, H, eps, dtype) -> torch.Tensor:
-    """Per head o / rms(o) * w * silu(z): fp32 [T, H, Dv] -> [T, H*Dv]."""
+def rms_gate(o, z, w, H, eps, dtype, gate="silu", scale=1.0,
+             out=None) -> torch.Tensor:
+    """Per head scale * o / rms(o) * w * act(z): fp32 [T, H, Dv] ->
+    [T, H*Dv]. ``w`` [Dv] serves every head, [H*Dv] gives each head its
+    own; ``gate`` "silu" or "sigmoid"; ``out`` may be a column block of
+    a wider buffer."""
+    assert gate in ("silu", "sigmoid")
     if o.is_cuda:
-        out = torch.empty(o.shape[0], o.shape[1] * o.shape[2], dtype=dtype,
-                          device=o.device)
-        _seq_kernels().rms_gate(out, o, z, w, H, eps)
+        if out is None:
+            out = torch.empty(o.shape[0], o.shape[1] * o.shape[2],
+                              dtype=dtype, device=o.device)
+        _seq_kernels().rms_gate(out, o, z, w, H, eps, gate == "sigmoid",
+                                float(scale))
         return out
     from gllm_amd.ops import gdn_ref
-    return gdn_ref.rms_gate(o, z, w, H, eps, dtype)
+    return gdn_ref.rms_gate(o, z, w, H, eps, dtype, gate, scale, out)
+
+
+def general_delta_rule(r, k, v, w_logit, a_logit, w0, decay_scale, state,
+                       slots, has_init, query_start_loc,
+                       max_query_len=0) -> torch.Tensor:
+    """Ragged generalized delta rule with per-channel decay and removal
+    (prompt portions and decode tokens in one launch). Per head, with
+    w = exp(-decay_scale * sigmoid(w_logit + w0)), a = sigmoid(a_logit),
+    u = k / sqrt(|k|^2 + 1e-6):
+        S <- diag(w) S - (a u)(u^T S) + k v^T,   o = S^T r
+    fp32 state [slots, H, D, Dv] in place; decay, removal rate and the
+    unit key are formed in fp32 from the projections. Returns fp32
+    [T, H, Dv]."""
+    if r.is_cuda:
+        H, _, Dv = state.shape[1:]
+        o = torch.empty(r.shape[0], H, Dv, dtype=torch.float32,
+                        device=r.device)
+        _seq_kernels().general_delta_rule(
+            o, r, k, v, w_logit, a_logit, w0, float(decay_scale), state,
+            slots, has_init, query_start_loc, int(max_query_len))
+        return o
+    from gllm_amd.ops import gdn_ref
+    return gdn_ref.general_delta_rule(r, k, v, w_logit, a_logit, w0,
+                                      decay_scale, state, slots, has_init,
+                                      query_start_loc)
+
+
+def token_shift(h, mu, state, slots, has_init, query_start_loc):
+    """Ragged token shift h_t + (h_(t-1) - h_t) * mu: the row before a
+    portion's first comes from ``state`` [slots, width] (zeros when the
+    sequence starts here), which is left at the portion's last incoming
+    row."""
+    if h.is_cuda:
+        out = torch.empty_like(h)
+        _seq_kernels().token_shift(out, h, mu, state, slots, has_init,
+                                   query_start_loc)
+        return out
+    return torch_ref.token_shift(h, mu, state, slots, has_init,
+                                 query_start_loc)

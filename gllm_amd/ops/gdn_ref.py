@@ -225,11 +225,12 @@ def rmsnorm_gated(x: torch.Tensor, z: torch.Tensor, weight: torch.Tensor,
 # ------------------------------------------------------------------
 # ragged (varlen) forms over per-slot state pools: the CPU path and the
 # kernel oracle of ops.causal_conv_silu / delta_rule_varlen / rms_gate
-def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc):
-    """Short causal depthwise conv + silu over a ragged batch. ``x``
-    [T, C], ``w`` [C, taps] (last tap = current token), ``conv_state``
-    [slots, C, taps-1] holds each sequence's previous inputs and is
-    rolled forward in place."""
+def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc,
+                     activation=True):
+    """Short causal depthwise conv (+ silu unless ``activation`` is
+    False) over a ragged batch. ``x`` [T, C], ``w`` [C, taps] (last tap
+    = current token), ``conv_state`` [slots, C, taps-1] holds each
+    sequence's previous inputs and is rolled forward in place."""
     taps = w.shape[1]
     qsl = query_start_loc.tolist()
     out = torch.empty(x.shape, dtype=x.dtype)
@@ -243,7 +244,7 @@ def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc):
         acc = torch.zeros(e - s, x.shape[1], dtype=torch.float32)
         for tap in range(taps):
             acc += seq[tap:tap + e - s].float() * w[:, tap].float()
-        out[s:e] = F.silu(acc).to(x.dtype)
+        out[s:e] = (F.silu(acc) if activation else acc).to(x.dtype)
         if taps > 1:
             conv_state[slot] = seq[seq.shape[0] - (taps - 1):].t()
     return out
@@ -283,9 +284,51 @@ def delta_rule_varlen(q, k, v, a, b, A_log, dt_bias, state, slots,
     return out
 
 
-def rms_gate(o, z, w, H, eps, dtype):
-    """Per head: o / rms(o) * w * silu(z); o fp32 [T, H, Dv]."""
+def rms_gate(o, z, w, H, eps, dtype, gate="silu", scale=1.0, out=None):
+    """Per head: scale * o / rms(o) * w * act(z); o fp32 [T, H, Dv], w
+    [Dv] (shared by the heads) or [H * Dv], act = silu or sigmoid."""
     T = o.shape[0]
     of = o.float().reshape(T, H, -1)
-    of = of * torch.rsqrt((of * of).mean(-1, keepdim=True) + eps) * w.float()
-    return (of.reshape(T, -1) * F.silu(z.float())).to(dtype)
+    of = of * torch.rsqrt((of * of).mean(-1, keepdim=True) + eps)
+    wf = w.float()
+    of = of * (wf if wf.numel() == of.shape[2] else wf.view(H, -1))
+    zf = z.float()
+    act = F.silu(zf) if gate == "silu" else torch.sigmoid(zf)
+    res = (of.reshape(T, -1) * act * scale).to(dtype)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+def general_delta_rule(r, k, v, w_logit, a_logit, w0, decay_scale, state,
+                       slots, has_init, query_start_loc):
+    """Token-by-token generalized delta rule over a ragged batch; fp32
+    state [slots, H, D, Dv] (key x value) in place. Per head, with
+    w = exp(-decay_scale * sigmoid(w_logit + w0)), a = sigmoid(a_logit)
+    and the unit key u = k / sqrt(|k|^2 + 1e-6):
+        S <- diag(w) S - (a u)(u^T S) + k v^T,   o = S^T r
+    (both subtracted and decayed terms read the old S). r, k, w_logit,
+    a_logit [T, H*D], v [T, H*Dv], w0 [H*D]; returns fp32 [T, H, Dv]."""
+    H, D, Dv = state.shape[1:]
+    T = r.shape[0]
+    rf = r.float().reshape(T, H, D)
+    kf = k.float().reshape(T, H, D)
+    vf = v.float().reshape(T, H, Dv)
+    w = torch.exp(-decay_scale * torch.sigmoid(
+        w_logit.float() + w0.float())).reshape(T, H, D)
+    a = torch.sigmoid(a_logit.float()).reshape(T, H, D)
+    u = kf / torch.sqrt((kf * kf).sum(-1, keepdim=True) + 1e-6)
+    out = torch.empty(T, H, Dv, dtype=torch.float32)
+    qsl = query_start_loc.tolist()
+    for i, slot in enumerate(slots.tolist()):
+        S = state[slot].clone() if bool(has_init[i]) \
+            else torch.zeros(H, D, Dv)
+        for t in range(qsl[i], qsl[i + 1]):
+            uS = torch.einsum("hkv,hk->hv", S, u[t])
+            S = S * w[t, :, :, None] \
+                - (a[t] * u[t])[:, :, None] * uS[:, None, :] \
+                + kf[t, :, :, None] * vf[t, :, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", S, rf[t])
+        state[slot] = S
+    return out

@@ -288,17 +288,96 @@ def residual_layernorm(x: torch.Tensor, y: torch.Tensor, w_post, b_post,
     return layernorm_f32(x, pre[0], pre[1], eps, y.dtype)
 
 
+def stream_rmsnorm(x, y, w_post, eps, mult=1.0, y_scale=1.0, y2=None,
+                   add=None, pre_w=None):
+    """fp32 stream x (in place): x += mult * RMSnorm(y_scale * (y + y2))
+    * w_post (skipped when ``y`` is None), then x += add (one fp32 row
+    for every token); returns RMSnorm(x) * pre_w in pre_w's dtype when
+    ``pre_w`` is given."""
+    if y is not None:
+        z = y.float()
+        if y2 is not None:
+            z = z + y2.float()
+        z = z * y_scale
+        z = z * torch.rsqrt((z * z).mean(-1, keepdim=True) + eps)
+        x.add_(z * w_post.float() * mult)
+    if add is not None:
+        x.add_(add.float())
+    if pre_w is None:
+        return None
+    h = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+    return (h * pre_w.float()).to(pre_w.dtype)
+
+
+def token_shift(h, mu, state, slots, has_init, query_start_loc):
+    """Ragged token shift: row t becomes h_t + (h_(t-1) - h_t) * mu with
+    h_(t-1) the row before it as it came in; a portion's first row
+    looks at ``state[slot]`` (zeros for a sequence's first token), and
+    the state is left at the portion's last incoming row."""
+    out = torch.empty_like(h)
+    qsl = query_start_loc.tolist()
+    muf = mu.float()
+    for b, slot in enumerate(slots.tolist()):
+        s, e = qsl[b], qsl[b + 1]
+        if e <= s:
+            continue
+        first = state[slot].to(h.dtype) if bool(has_init[b]) \
+            else h.new_zeros(h.shape[1])
+        prev = torch.cat([first[None], h[s:e - 1]]).float()
+        cur = h[s:e].float()
+        out[s:e] = (cur + (prev - cur) * muf).to(h.dtype)
+        state[slot] = h[e - 1].to(state.dtype)
+    return out
+
+
+def gelu_tanh_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """gelu_tanh(x[:, :d]) * x[:, d:] with the tanh form of gelu."""
+    d = x.shape[-1] // 2
+    a = x[..., :d].float()
+    return (torch.nn.functional.gelu(a, approximate="tanh") *
+            x[..., d:].float()).to(x.dtype)
+
+
+def sigmoid_group_topk(logits, correction, topk, n_group, keep, scale):
+    """Sigmoid routing with group limits: s = sigmoid(logits); the
+    choice runs on s + correction among the experts of the ``keep``
+    groups (of ``n_group`` equal neighbour groups) whose two best choice
+    scores sum highest, everything else counting as -inf; the weights
+    are the chosen s over their sum (+ 1e-20), times ``scale``.
+    n_group <= 1: no group limit. Ties go to the lower index."""
+    T, E = logits.shape
+    s = torch.sigmoid(logits.float())
+    sel = s + correction.float() if correction is not None else s.clone()
+    if n_group > 1:
+        per = E // n_group
+        g = sel.view(T, n_group, per)
+        gscore = g.topk(min(2, per), dim=-1)[0].sum(-1)
+        order = torch.sort(gscore, dim=-1, descending=True, stable=True)[1]
+        mask = torch.zeros(T, n_group, dtype=torch.bool)
+        mask.scatter_(1, order[:, :keep], True)
+        mask = mask.unsqueeze(-1).expand(T, n_group, per).reshape(T, E)
+        sel = sel.masked_fill(~mask, float("-inf"))
+    ids = torch.sort(sel, dim=-1, descending=True, stable=True)[1][:, :topk]
+    w = s.gather(1, ids)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+    return w, ids.to(torch.int32)
+
+
 def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
                        mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
                        half_layout=False, norm_last=False, do_norm=True,
-                       v_freqs=None):
+                       v_freqs=None, norm_span=False, v_unit=False):
     """Per-head RMS norm (plain weight, or none when the weight is None)
     + rotary on q (in place) and k; k, v land in the paged cache rows
     ``slot_mapping``. ``k`` None: a layer that reads another layer's
     cache. ``half_layout``: dimension i pairs with i + rot_dims/2
     instead of (2i, 2i+1); ``norm_last``: rotate first, then norm;
     ``do_norm`` False: rotary only. ``v_freqs`` [Dv/2]: every value row
-    is turned by its own position over all of Dv before it is stored."""
+    is turned by its own position over all of Dv before it is stored.
+    ``norm_span``: the RMS is taken over all heads of a token's row at
+    once and the weights cover the row ([heads * D]). ``v_unit``: every
+    value head is brought to unit RMS (eps, no weight) before the
+    store."""
     T = q.shape[0]
     ang = positions[:T].double()[:, None] * freqs.double()[None, :rot_dims // 2]
     cos = (torch.cos(ang).float() * mag)[:, None, :]
@@ -308,6 +387,10 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
     def norm(xf, w):
         if not do_norm:
             return xf
+        if norm_span:
+            ms = (xf * xf).mean((-2, -1), keepdim=True)
+            xf = xf * torch.rsqrt(ms + eps)
+            return xf if w is None else xf * w.float().view(xf.shape[1:])
         xf = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
         return xf if w is None else xf * w.float()
 
@@ -334,6 +417,9 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
     vc = v_cache.view(-1, G, Dv)
     kc[rows] = prep(k, k_w, G).to(k_cache.dtype)
     vv = v.reshape(T, G, Dv)
+    if v_unit:
+        vf = vv.float()
+        vv = vf * torch.rsqrt((vf * vf).mean(-1, keepdim=True) + eps)
     if v_freqs is not None:
         vv = rotate_scale_rows(vv.reshape(T, G * Dv), positions, v_freqs,
                                G, Dv, 1.0, 1.0, half_layout
