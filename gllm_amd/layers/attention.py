@@ -158,6 +158,12 @@ class WindowAttention(nn.Module):
         half = bool(getattr(self.rotary, "half_layout", False))
         vrot = self.value_rotary
         vfreqs = vrot.freqs if vrot is not None else None
+        q_out = None
+        if self.norm_span:
+            # every head reads the whole incoming row: queries land in
+            # a buffer of their own
+            q_out = torch.empty(T, self.num_heads * self.head_dim,
+                                dtype=q.dtype, device=q.device)
         if self.owns_kv:
             ops.qk_norm_rope_store(
                 q, k, v, self.q_norm, self.k_norm, fctx.positions,
@@ -165,14 +171,18 @@ class WindowAttention(nn.Module):
                 self.num_heads, self.num_kv_heads, self.head_dim,
                 self.v_head_dim, self.eps, half_layout=half,
                 do_norm=self.qk_norm, v_freqs=vfreqs,
-                norm_span=self.norm_span, v_unit=self.value_unit_norm)
+                norm_span=self.norm_span, v_unit=self.value_unit_norm,
+                q_out=q_out)
         else:
             ops.qk_norm_rope_store(
                 q, None, None, self.q_norm, None, fctx.positions,
                 fctx.slot_mapping, freqs, mag, rot_dims, None, None,
                 self.num_heads, self.num_kv_heads, self.head_dim,
                 self.v_head_dim, self.eps, half_layout=half,
-                do_norm=self.qk_norm, norm_span=self.norm_span)
+                do_norm=self.qk_norm, norm_span=self.norm_span,
+                q_out=q_out)
+        if q_out is not None:
+            q = q_out
         o = ops.window_attention(
             q, gate, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
             fctx.query_start_loc, self.scale, self.window,

@@ -121,7 +121,8 @@ class TokenShift(nn.Module):
         sid = self.ssm_layer_id if ssm_layer_id is None else ssm_layer_id
         slots, init = state_rows(fctx, h.shape[0], h.device)
         return ops.token_shift(h, self.mu, fctx.ssm_pool.shift_state[sid],
-                               slots, init, fctx.query_start_loc)
+                               slots, init, fctx.query_start_loc,
+                               fctx.max_query_len)
 
 
 class GeneralDeltaRule(nn.Module):

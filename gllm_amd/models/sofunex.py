@@ -193,7 +193,7 @@ class DenseGLU(nn.Module):
         self.down = RowParallelLinear(ff, width, params_dtype=dtype)
 
     def forward(self, h: torch.Tensor):
-        return self.down(ops.gelu_tanh_and_mul(self.in_proj(h))), None
+        return self.down(ops.gated_act_mul(self.in_proj(h), "gelu_tanh")), None
 
 
 class GroupRoutedExperts(nn.Module):
@@ -242,7 +242,7 @@ class GroupRoutedExperts(nn.Module):
         y = self.experts.forward_routed(h, weights, ids)
         if not self.shared_ff:
             return y, None
-        return y, self.shared_down(ops.silu_and_mul(self.shared_in(h)))
+        return y, self.shared_down(ops.gated_act_mul(self.shared_in(h), "silu"))
 
 
 class SofunexLayer(nn.Module):

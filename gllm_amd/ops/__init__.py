@@ -812,14 +812,17 @@ def stream_rmsnorm(x: torch.Tensor, y, w_post, eps: float,
                                     add, pre_w)
 
 
-def gelu_tanh_and_mul(x: torch.Tensor) -> torch.Tensor:
-    """x [rows, 2d] = gate | up -> gelu_tanh(gate) * up."""
+def gated_act_mul(x: torch.Tensor, act: str = "silu") -> torch.Tensor:
+    """x [rows, 2d] = gate | up -> act(gate) * up with act "silu" or
+    "gelu_tanh"; any d, rows may be strided (bf16 or fp32)."""
+    assert act in ("silu", "gelu_tanh")
     if x.is_cuda:
-        d = x.shape[-1] // 2
-        out = torch.empty(x.shape[:-1] + (d,), dtype=x.dtype,
+        out = torch.empty(x.shape[0], x.shape[1] // 2, dtype=x.dtype,
                           device=x.device)
-        _seq_kernels().gelu_tanh_and_mul(out, x)
+        _seq_kernels().gated_act_mul(out, x, 0 if act == "silu" else 1)
         return out
+    if act == "silu":
+        return torch_ref.silu_and_mul(x)
     return torch_ref.gelu_tanh_and_mul(x)
 
 
@@ -846,7 +849,8 @@ def sigmoid_group_topk(logits: torch.Tensor, correction, topk: int,
 def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
                        mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
                        half_layout=False, norm_last=False, do_norm=True,
-                       v_freqs=None, norm_span=False, v_unit=False):
+                       v_freqs=None, norm_span=False, v_unit=False,
+                       q_out=None):
     """Fused per-head q/k RMS norm, rotary (per-pair frequency table
     ``freqs`` fp64, cos/sin scaled by ``mag``) and paged K/V store.
     q [T, H*D] is updated in place (may be a column slice of a merged
@@ -862,19 +866,20 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
     ``norm_span``: one RMS over all heads of a token's q (and of its k)
     with weights that cover the row ([H*D], [G*D]). ``v_unit``: each
     value head is divided by its RMS (eps inside the root, no weight)
-    before it is stored."""
+    before it is stored. ``q_out`` ([T, H*D]): the prepared queries go
+    there and q stays as it came (required with ``norm_span``)."""
     if q.is_cuda:
         _seq_kernels().qk_norm_rope_store(
             q, k, v, q_w, k_w, positions, slot_mapping, freqs, mag,
             rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
             bool(half_layout), bool(norm_last), bool(do_norm), v_freqs,
-            bool(norm_span), bool(v_unit))
+            bool(norm_span), bool(v_unit), q_out)
         return
     torch_ref.qk_norm_rope_store(q, k, v, q_w, k_w, positions,
                                  slot_mapping, freqs, mag, rot_dims,
                                  k_cache, v_cache, H, G, D, Dv, eps,
                                  half_layout, norm_last, do_norm, v_freqs,
-                                 norm_span, v_unit)
+                                 norm_span, v_unit, q_out)
 
 
 def rotate_scale_rows(x, positions, freqs, heads, D, sign=1.0, scale=1.0,
@@ -1138,7 +1143,8 @@ def general_delta_rule(r, k, v, w_logit, a_logit, w0, decay_scale, state,
                                       query_start_loc)
 
 
-def token_shift(h, mu, state, slots, has_init, query_start_loc):
+def token_shift(h, mu, state, slots, has_init, query_start_loc,
+                max_query_len=0):
     """Ragged token shift h_t + (h_(t-1) - h_t) * mu: the row before a
     portion's first comes from ``state`` [slots, width] (zeros when the
     sequence starts here), which is left at the portion's last incoming
@@ -1146,7 +1152,7 @@ def token_shift(h, mu, state, slots, has_init, query_start_loc):
     if h.is_cuda:
         out = torch.empty_like(h)
         _seq_kernels().token_shift(out, h, mu, state, slots, has_init,
-                                   query_start_loc)
+                                   query_start_loc, int(max_query_len))
         return out
     return torch_ref.token_shift(h, mu, state, slots, has_init,
                                  query_start_loc)

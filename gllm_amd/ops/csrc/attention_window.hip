@@ -13,7 +13,10 @@
 //                       rotation (or no norm at all), then q in place
 //                       and k, v scattered into the paged cache (v may
 //                       be k as projected; with a value frequency table
-//                       v is turned by its own position over all of Dv)
+//                       v is turned by its own position over all of Dv);
+//                       span norm: ONE RMS over all heads of the token's
+//                       q (k) row with row-sized weights; unit values:
+//                       each value head divided by its RMS on the way in
 //   window_attention    ragged batch (prompt portions beside single
 //                       decode tokens) over the paged cache: position i
 //                       sees j <= i with i - j < window or j < keep_first;
@@ -50,7 +53,8 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
     const long *__restrict__ slot_mapping, const double *__restrict__ freqs,
     float mag, int rot_dims, T *__restrict__ k_cache, T *__restrict__ v_cache,
     int H, int G, int D, int Dv, float eps, int half_layout, int norm_last,
-    int do_norm, const double *__restrict__ v_freqs) {
+    int do_norm, const double *__restrict__ v_freqs, int norm_span,
+    int v_unit, T *__restrict__ q_out, long q_out_stride) {
   extern __shared__ float buf[];
   const int t = blockIdx.x;
   const int y = blockIdx.y;
@@ -60,6 +64,17 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
     const long slot = slot_mapping[t];
     const T *src = v + (long)t * v_stride + (long)g * Dv;
     T *dst = v_cache + (slot * G + g) * Dv;
+    if (v_unit) {  // unit RMS per head (no rotation on this path)
+      float vs = 0.f;
+      for (int i = lane; i < Dv; i += QK_BLOCK) {
+        const float x = ScalarOps<T>::to_f32(src[i]);
+        vs += x * x;
+      }
+      const float vinv = 1.0f / sqrtf(wave_reduce_sum(vs) / Dv + eps);
+      for (int i = lane; i < Dv; i += QK_BLOCK)
+        dst[i] = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(src[i]) * vinv);
+      return;
+    }
     if (v_freqs == nullptr) {
       for (int i = lane; i < Dv; i += QK_BLOCK) dst[i] = src[i];
       return;
@@ -83,6 +98,8 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
   const T *src = is_q ? q + (long)t * q_stride + (long)y * D
                       : k + (long)t * k_stride + (long)(y - H) * D;
   const T *w = is_q ? q_w : k_w;
+  // span norm: the weights cover the row, this head reads its block
+  if (norm_span && w) w += (long)(is_q ? y : y - H) * D;
   float ss = 0.f;
   for (int i = lane; i < D; i += QK_BLOCK) {
     const float x = ScalarOps<T>::to_f32(src[i]);
@@ -91,8 +108,21 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
   }
   __syncthreads();
   if (do_norm && !norm_last) {
+    int n = D;
+    if (norm_span) {
+      // every head of the row sums the whole row, in the same order, so
+      // all heads of a token scale by the same number (the host makes q
+      // land in a buffer of its own: the row stays as it came in)
+      const T *row = is_q ? q + (long)t * q_stride : k + (long)t * k_stride;
+      n = (is_q ? H : G) * D;
+      ss = 0.f;
+      for (int i = lane; i < n; i += QK_BLOCK) {
+        const float x = ScalarOps<T>::to_f32(row[i]);
+        ss += x * x;
+      }
+    }
     ss = wave_reduce_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / D + eps);
+    const float inv = 1.0f / sqrtf(ss / n + eps);
     for (int i = lane; i < D; i += QK_BLOCK)
       buf[i] = buf[i] * inv * (w ? ScalarOps<T>::to_f32(w[i]) : 1.0f);
     __syncthreads();
@@ -119,7 +149,7 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
       buf[i] = buf[i] * inv * (w ? ScalarOps<T>::to_f32(w[i]) : 1.0f);
     __syncthreads();
   }
-  T *dst = is_q ? q + (long)t * q_stride + (long)y * D
+  T *dst = is_q ? q_out + (long)t * q_out_stride + (long)y * D
                 : k_cache + (slot_mapping[t] * G + (y - H)) * D;
   for (int i = lane; i < D; i += QK_BLOCK)
     dst[i] = ScalarOps<T>::from_f32(buf[i]);
@@ -286,14 +316,34 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
                         c10::optional<torch::Tensor> v_cache, long H, long G,
                         long D, long Dv, double eps, bool half_layout,
                         bool norm_last, bool do_norm,
-                        c10::optional<torch::Tensor> v_freqs) {
+                        c10::optional<torch::Tensor> v_freqs, bool norm_span,
+                        bool v_unit, c10::optional<torch::Tensor> q_out) {
   const long T = q.size(0);
+  // span norm: other heads still read the incoming row while one head
+  // writes, so the result needs a buffer of its own
+  TORCH_CHECK(!norm_span || q_out.has_value(),
+              "span norm writes q out of place");
+  void *qop = q.data_ptr();
+  long qos = q.stride(0);
+  if (q_out.has_value()) {
+    TORCH_CHECK(q_out->is_cuda() && rows_ok(*q_out) &&
+                q_out->sizes() == q.sizes() &&
+                q_out->scalar_type() == q.scalar_type() &&
+                q_out->data_ptr() != q.data_ptr());
+    qop = q_out->data_ptr();
+    qos = q_out->stride(0);
+  }
+  TORCH_CHECK(!norm_span || (do_norm && !norm_last),
+              "span norm runs before the rotation");
+  TORCH_CHECK(!v_unit || !v_freqs.has_value(),
+              "unit values and rotated values do not combine");
   if (T == 0) return;
   const auto st = q.scalar_type();
   TORCH_CHECK(q.is_cuda() && rows_ok(q) && q.size(1) == H * D);
   const void *qwp = nullptr;
   if (q_w.has_value()) {
-    TORCH_CHECK(q_w->scalar_type() == st && q_w->numel() == D &&
+    TORCH_CHECK(q_w->scalar_type() == st &&
+                q_w->numel() == (norm_span ? H * D : D) &&
                 q_w->is_contiguous());
     qwp = q_w->data_ptr();
   }
@@ -316,7 +366,8 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
     TORCH_CHECK(rows_ok(*v) && v->size(0) == T && v->size(1) == G * Dv &&
                 v->scalar_type() == st);
     if (k_w.has_value()) {
-      TORCH_CHECK(k_w->scalar_type() == st && k_w->numel() == D &&
+      TORCH_CHECK(k_w->scalar_type() == st &&
+                  k_w->numel() == (norm_span ? G * D : D) &&
                   k_w->is_contiguous());
       kwp = k_w->data_ptr();
     }
@@ -350,7 +401,8 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
                      freqs.data_ptr<double>(), (float)mag, (int)rot_dims,    \
                      (TT *)kcp, (TT *)vcp, (int)H, (int)G, (int)D, (int)Dv,  \
                      (float)eps, half_layout ? 1 : 0, norm_last ? 1 : 0,     \
-                     do_norm ? 1 : 0, vfp)
+                     do_norm ? 1 : 0, vfp, norm_span ? 1 : 0, v_unit ? 1 : 0, \
+                     (TT *)qop, qos)
   if (st == at::kBFloat16) RUN(__hip_bfloat16);
   else if (st == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "qk_norm_rope_store: bf16 or fp32");

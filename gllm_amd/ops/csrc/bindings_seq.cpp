@@ -24,7 +24,8 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
                         c10::optional<torch::Tensor> v_cache, long H, long G,
                         long D, long Dv, double eps, bool half_layout,
                         bool norm_last, bool do_norm,
-                        c10::optional<torch::Tensor> v_freqs);
+                        c10::optional<torch::Tensor> v_freqs, bool norm_span,
+                        bool v_unit, c10::optional<torch::Tensor> q_out);
 void rotate_scale_rows(torch::Tensor out, torch::Tensor x,
                        torch::Tensor positions, torch::Tensor freqs,
                        long heads, long D, double sign, double scale,
@@ -79,7 +80,8 @@ bool window_attention_decode(torch::Tensor out, torch::Tensor q,
                              double softcap);
 void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                       torch::Tensor conv_state, torch::Tensor slots,
-                      torch::Tensor has_init, torch::Tensor query_start_loc);
+                      torch::Tensor has_init, torch::Tensor query_start_loc,
+                      bool activation);
 void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                        torch::Tensor v, torch::Tensor a, torch::Tensor b,
                        torch::Tensor A_log, torch::Tensor dt_bias,
@@ -87,7 +89,30 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                        torch::Tensor has_init, torch::Tensor query_start_loc,
                        double q_scale, long max_query_len);
 void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
-              torch::Tensor w, long H, double eps);
+              torch::Tensor w, long H, double eps, bool sigmoid_gate,
+              double scale);
+void token_shift(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
+                 torch::Tensor state, torch::Tensor slots,
+                 torch::Tensor has_init, torch::Tensor query_start_loc,
+                 long max_query_len);
+void general_delta_rule(torch::Tensor o, torch::Tensor r, torch::Tensor k,
+                        torch::Tensor v, torch::Tensor w_logit,
+                        torch::Tensor a_logit, torch::Tensor w0,
+                        double decay_scale, torch::Tensor state,
+                        torch::Tensor slots, torch::Tensor has_init,
+                        torch::Tensor query_start_loc, long max_query_len);
+void stream_rmsnorm(torch::Tensor x, c10::optional<torch::Tensor> y,
+                    c10::optional<torch::Tensor> y2,
+                    c10::optional<torch::Tensor> w_post,
+                    c10::optional<torch::Tensor> add,
+                    c10::optional<torch::Tensor> h,
+                    c10::optional<torch::Tensor> w_pre, double eps,
+                    double mult, double y_scale);
+void gated_act_mul(torch::Tensor out, torch::Tensor x, long act);
+void sigmoid_group_topk(torch::Tensor weights, torch::Tensor ids,
+                        torch::Tensor logits,
+                        c10::optional<torch::Tensor> correction,
+                        long n_group, long keep, double scale);
 // shared with the full extension (skinny_gemm.hip, moe.hip,
 // elementwise.hip): what ops.linear / FusedMoE dispatch to in bf16
 void skinny_gemm(torch::Tensor out, torch::Tensor x, torch::Tensor w,
@@ -141,7 +166,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "ragged short causal conv + silu with per-slot state");
   m.def("delta_rule_varlen", &delta_rule_varlen,
         "ragged gated delta rule, fp32 state in registers");
-  m.def("rms_gate", &rms_gate, "o / rms(o) * w * silu(z) per head");
+  m.def("rms_gate", &rms_gate, "scale * o / rms(o) * w * act(z) per head");
+  m.def("token_shift", &token_shift,
+        "ragged token shift over the per-slot last-row state");
+  m.def("general_delta_rule", &general_delta_rule,
+        "ragged delta rule with per-channel decay and removal rate");
+  m.def("stream_rmsnorm", &stream_rmsnorm,
+        "x += mult * RMS(y) w_post (+ add); h = RMS(x) w_pre");
+  m.def("gated_act_mul", &gated_act_mul, "act(x[:d]) * x[d:], silu or gelu");
+  m.def("sigmoid_group_topk", &sigmoid_group_topk,
+        "sigmoid router with correction and group limits");
   m.def("skinny_gemm", &skinny_gemm,
         "decode-regime weight-streaming GEMM (M<=256)");
   m.def("silu_and_mul", &silu_and_mul, "silu(x[:d]) * x[d:]");

@@ -20,7 +20,17 @@
 //                      waves never meet at a barrier: the state column
 //                      block lives in registers for the whole portion.
 //                      Norms and gates come from a per-token pre-pass.
-//   rms_gate           o / rms(o) * w * silu(z) per head
+//   rms_gate           scale * o / rms(o) * w * act(z) per head, act silu
+//                      or sigmoid, w shared by the heads or one per head
+//   token_shift        h_t + (h_(t-1) - h_t) * mu over a ragged batch; the
+//                      row before a portion comes from the per-slot state
+//   general_delta_rule per (sequence, head): for each token
+//                        d = k^T S;  S <- diag(w) S - ak d^T + k v^T;
+//                        o = S^T r
+//                      with w = exp(-c sigmoid(.)) per key channel and
+//                      ak = sigmoid(.) k / (|k|^2 + 1e-6) (removal rate on
+//                      the unit key, folded) from a per-token pre-pass;
+//                      same lane layout as delta_rule_varlen
 //
 // State layouts: conv [slots, C, taps-1] (oldest first), recurrent
 // [slots, H, Dk, Dv] fp32.
@@ -50,7 +60,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
     T *__restrict__ out, const T *__restrict__ x, long x_stride,
     const T *__restrict__ w, const T *__restrict__ state,
     const long *__restrict__ slots, const int *__restrict__ has_init,
-    const int *__restrict__ qsl, int B, int C, int taps) {
+    const int *__restrict__ qsl, int B, int C, int taps, int act) {
   const int t = blockIdx.x;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
@@ -69,7 +79,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
     acc += xv * ScalarOps<T>::to_f32(w[(long)c * taps + tap]);
   }
   // the activation output feeds 16-bit consumers in bf16 serving
-  out[(long)t * C + c] = ScalarOps<T>::from_f32(silu_f(acc));
+  out[(long)t * C + c] = ScalarOps<T>::from_f32(act ? silu_f(acc) : acc);
 }
 
 // 8 channels per thread, 16 B accesses (C % 8 == 0, aligned rows);
@@ -80,7 +90,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu8_kernel(
     T *__restrict__ out, const T *__restrict__ x, long x_stride,
     const T *__restrict__ w, const T *__restrict__ state,
     const long *__restrict__ slots, const int *__restrict__ has_init,
-    const int *__restrict__ qsl, int B, int C) {
+    const int *__restrict__ qsl, int B, int C, int act) {
   const int t = blockIdx.x;
   const int c0 = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (c0 >= C) return;
@@ -109,8 +119,10 @@ __global__ __launch_bounds__(256) void causal_conv_silu8_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += xv[e] * wf[e * TAPS + tap];
   }
+  if (act) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = silu_f(acc[e]);
+    for (int e = 0; e < 8; ++e) acc[e] = silu_f(acc[e]);
+  }
   st8<T>(out + (long)t * C + c0, acc);
 }
 
@@ -465,12 +477,17 @@ __global__ __launch_bounds__(256) void delta_rule_tiled_kernel(
   }
 }
 
-// grid (tokens * H); block 64: out = o / rms(o) * w * silu(z)
+DEV_INLINE float gate_act(float z, int sig) {
+  return sig ? 1.0f / (1.0f + expf(-z)) : silu_f(z);
+}
+
+// grid (tokens * H); block 64: out = scale * o / rms(o) * w * act(z);
+// w_hs = 0: one weight row for all heads, Dv: a row per head
 template <typename T>
 __global__ __launch_bounds__(64) void rms_gate_kernel(
-    T *__restrict__ out, const float *__restrict__ o,
+    T *__restrict__ out, long out_stride, const float *__restrict__ o,
     const T *__restrict__ z, long z_stride, const T *__restrict__ w,
-    int H, int Dv, float eps) {
+    int w_hs, int H, int Dv, float eps, int sig, float scale) {
   const long th = blockIdx.x;
   const long t = th / H;
   const int h = th % H;
@@ -478,11 +495,12 @@ __global__ __launch_bounds__(64) void rms_gate_kernel(
   float ss = 0.f;
   for (int d = threadIdx.x; d < Dv; d += 64) ss += orow[d] * orow[d];
   ss = wave_reduce_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / Dv + eps);
+  const float inv = scale / sqrtf(ss / Dv + eps);
   for (int d = threadIdx.x; d < Dv; d += 64) {
     const float zz = ScalarOps<T>::to_f32(z[t * z_stride + (long)h * Dv + d]);
-    out[th * Dv + d] = ScalarOps<T>::from_f32(
-        orow[d] * inv * ScalarOps<T>::to_f32(w[d]) * silu_f(zz));
+    out[t * out_stride + (long)h * Dv + d] = ScalarOps<T>::from_f32(
+        orow[d] * inv * ScalarOps<T>::to_f32(w[(long)h * w_hs + d]) *
+        gate_act(zz, sig));
   }
 }
 
@@ -490,9 +508,9 @@ __global__ __launch_bounds__(64) void rms_gate_kernel(
 // grid ceil(rows / (256 / LPR)), block 256
 template <typename T, int LPR>
 __global__ __launch_bounds__(256) void rms_gate8_kernel(
-    T *__restrict__ out, const float *__restrict__ o,
+    T *__restrict__ out, long out_stride, const float *__restrict__ o,
     const T *__restrict__ z, long z_stride, const T *__restrict__ w,
-    int H, long rows, float eps) {
+    int w_hs, int H, long rows, float eps, int sig, float scale) {
   constexpr int Dv = LPR * 8;
   const long th = (long)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
   const int d0 = (threadIdx.x % LPR) * 8;
@@ -506,12 +524,197 @@ __global__ __launch_bounds__(256) void rms_gate8_kernel(
 #pragma unroll
   for (int e = 0; e < 8; ++e) ss += of[e] * of[e];
   ss = group_reduce_sum<LPR>(ss);
-  const float inv = 1.0f / sqrtf(ss / Dv + eps);
+  const float inv = scale / sqrtf(ss / Dv + eps);
   ld8<T>(z + t * z_stride + (long)h * Dv + d0, zf);
-  ld8<T>(w + d0, wf);
+  ld8<T>(w + (long)h * w_hs + d0, wf);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) of[e] = of[e] * inv * wf[e] * silu_f(zf[e]);
-  if (ok) st8<T>(out + th * Dv + d0, of);
+  for (int e = 0; e < 8; ++e)
+    of[e] = of[e] * inv * wf[e] * gate_act(zf[e], sig);
+  if (ok) st8<T>(out + t * out_stride + (long)h * Dv + d0, of);
+}
+
+// ------------------------------------------------------------------
+// Token shift. grid (tokens, ceil(W / (256 * EPT))), EPT = 8 (16 B
+// accesses) or 1. Row t of sequence b reads row t - 1 of the same
+// portion, or the slot's state row when it opens the portion (zeros when
+// the sequence starts here). `store` != 0 (every portion is one token):
+// the same thread then leaves its incoming values in the state, so one
+// launch does both; longer portions roll the state in a second launch
+// (another workgroup may still have to read the old row).
+template <typename T, int EPT>
+__global__ __launch_bounds__(256) void token_shift_kernel(
+    T *__restrict__ out, const T *__restrict__ h, long h_stride,
+    const T *__restrict__ mu, T *__restrict__ state,
+    const long *__restrict__ slots, const int *__restrict__ has_init,
+    const int *__restrict__ qsl, int B, int W, int store) {
+  const int t = blockIdx.x;
+  const int c0 = (blockIdx.y * 256 + threadIdx.x) * EPT;
+  if (c0 >= W) return;
+  const int b = find_seq(qsl, B, t);
+  const bool first = t == qsl[b];
+  T *st = state + (long)slots[b] * W + c0;
+  float cur[EPT], prev[EPT], m[EPT];
+  if (EPT == 8) {
+    ld8<T>(h + (long)t * h_stride + c0, cur);
+    ld8<T>(mu + c0, m);
+    if (!first) ld8<T>(h + (long)(t - 1) * h_stride + c0, prev);
+    else if (has_init[b] != 0) ld8<T>(st, prev);
+    else {
+#pragma unroll
+      for (int e = 0; e < EPT; ++e) prev[e] = 0.f;
+    }
+  } else {
+    cur[0] = ScalarOps<T>::to_f32(h[(long)t * h_stride + c0]);
+    m[0] = ScalarOps<T>::to_f32(mu[c0]);
+    prev[0] = !first ? ScalarOps<T>::to_f32(h[(long)(t - 1) * h_stride + c0])
+              : has_init[b] != 0 ? ScalarOps<T>::to_f32(st[0]) : 0.f;
+  }
+  float res[EPT];
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) res[e] = cur[e] + (prev[e] - cur[e]) * m[e];
+  if (EPT == 8) {
+    st8<T>(out + (long)t * W + c0, res);
+    if (store) st8<T>(st, cur);
+  } else {
+    out[(long)t * W + c0] = ScalarOps<T>::from_f32(res[0]);
+    if (store) st[0] = ScalarOps<T>::from_f32(cur[0]);
+  }
+}
+
+// grid (B, ceil(W / 256)): state[slot] <- last incoming row of the portion
+template <typename T>
+__global__ __launch_bounds__(256) void shift_state_kernel(
+    T *__restrict__ state, const T *__restrict__ h, long h_stride,
+    const long *__restrict__ slots, const int *__restrict__ qsl, int W) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= W || qsl[b + 1] <= qsl[b]) return;
+  state[(long)slots[b] * W + c] = h[(long)(qsl[b + 1] - 1) * h_stride + c];
+}
+
+// ------------------------------------------------------------------
+// Per-token operands of the generalized delta rule, once per (token,
+// head) instead of once per wave that needs them:
+//   prep[t, 0, h, i] = w  = exp(-c * sigmoid(w_logit + w0))
+//   prep[t, 1, h, i] = ak = sigmoid(a_logit) * k / (|k|^2 + 1e-6)
+// (removal rate times the unit key, times the unit key's own 1/|k|, so
+// the recurrence takes d = k^T S on the raw key). grid (tokens, H), block 64.
+template <typename T>
+__global__ __launch_bounds__(64) void general_delta_prep_kernel(
+    float *__restrict__ prep, const T *__restrict__ k, long k_stride,
+    const T *__restrict__ wl, long wl_stride, const T *__restrict__ al,
+    long al_stride, const T *__restrict__ w0, int H, int D, float c) {
+  const long t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const T *kr = k + t * k_stride + (long)h * D;
+  float ss = 0.f;
+  for (int i = lane; i < D; i += 64) {
+    const float kv = ScalarOps<T>::to_f32(kr[i]);
+    ss += kv * kv;
+  }
+  const float ik2 = 1.0f / (wave_reduce_sum(ss) + 1e-6f);
+  float *pw = prep + (t * 2 * H + h) * D;
+  float *pa = pw + (long)H * D;
+  for (int i = lane; i < D; i += 64) {
+    const float z = ScalarOps<T>::to_f32(wl[t * wl_stride + (long)h * D + i]) +
+                    ScalarOps<T>::to_f32(w0[(long)h * D + i]);
+    pw[i] = expf(-c / (1.0f + expf(-z)));
+    const float a = 1.0f / (1.0f + expf(-ScalarOps<T>::to_f32(
+                                     al[t * al_stride + (long)h * D + i])));
+    pa[i] = a * ScalarOps<T>::to_f32(kr[i]) * ik2;
+  }
+}
+
+// grid (B, H, ceil(Dv / 64)), block 256 = 4 independent waves; lane layout
+// of delta_rule_varlen_kernel: a wave owns 16 state columns, a quad of
+// lanes shares a column and splits the key axis in 4 slices of KP. Per token
+//   d = k^T S[:, col];  S[i, col] <- w_i S[i, col] - ak_i d + k_i v_col;
+//   o_col = r^T S[:, col]
+// PF: the next token's operands are loaded while this one is computed
+// (off for KP = 64, where they would not fit the register file).
+template <typename T, int KP, bool PF>
+__global__ __launch_bounds__(256) void general_delta_kernel(
+    float *__restrict__ o, const T *__restrict__ r, const T *__restrict__ k,
+    const T *__restrict__ v, long rkv_stride, const float *__restrict__ prep,
+    float *__restrict__ state, const long *__restrict__ slots,
+    const int *__restrict__ has_init, const int *__restrict__ qsl, int H,
+    int Dk, int Dv, int vec) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = blockIdx.z * 64 + wave * 16 + (lane >> 2);
+  const int part = lane & 3;
+  const int i0 = part * KP;
+  const int start = qsl[b], end = qsl[b + 1];
+  const bool live = col < Dv;
+  const int colc = live ? col : Dv - 1;  // clamp loads, mask stores
+  if (blockIdx.z * 64 + wave * 16 >= Dv) return;  // whole wave idle
+  if (start >= end) return;
+  const long PW = 2L * H * Dk;
+
+  float *sp = state + ((long)slots[b] * H + h) * Dk * Dv;
+  float S[KP];
+  const bool init = has_init[b] != 0;
+#pragma unroll
+  for (int i = 0; i < KP; ++i)
+    S[i] = (init && i0 + i < Dk) ? sp[(long)(i0 + i) * Dv + colc] : 0.f;
+
+  float kc[KP], rc[KP], wc[KP], ac[KP];
+  float vc;
+  auto load_tok = [&](long t, float *kk, float *rr, float *ww, float *aa,
+                      float &vv) {
+    load_slice<T, KP>(k + t * rkv_stride + (long)h * Dk, i0, Dk, vec, kk);
+    load_slice<T, KP>(r + t * rkv_stride + (long)h * Dk, i0, Dk, vec, rr);
+    const float *pp = prep + t * PW + (long)h * Dk;
+    load_slice<float, KP>(pp, i0, Dk, vec, ww);
+    load_slice<float, KP>(pp + (long)H * Dk, i0, Dk, vec, aa);
+    vv = ScalarOps<T>::to_f32(v[t * rkv_stride + (long)h * Dv + colc]);
+  };
+  if (PF) load_tok(start, kc, rc, wc, ac, vc);
+  for (int t = start; t < end; ++t) {
+    float kx[PF ? KP : 1], rx[PF ? KP : 1], wx[PF ? KP : 1], ax[PF ? KP : 1];
+    float vx = 0.f;
+    if (PF) {
+      // prefetch t + 1 (clamped: the last iteration re-reads row t)
+      load_tok(t + 1 < end ? t + 1 : t, kx, rx, wx, ax, vx);
+    } else {
+      load_tok(t, kc, rc, wc, ac, vc);
+    }
+    float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;  // 4 chains, not one
+#pragma unroll
+    for (int i = 0; i < KP; i += 4) {
+      d0 += S[i] * kc[i];
+      d1 += S[i + 1] * kc[i + 1];
+      d2 += S[i + 2] * kc[i + 2];
+      d3 += S[i + 3] * kc[i + 3];
+    }
+    const float d = quad_sum((d0 + d1) + (d2 + d3));
+    float e0 = 0.f, e1 = 0.f, e2 = 0.f, e3 = 0.f;
+#pragma unroll
+    for (int i = 0; i < KP; i += 4) {
+      S[i] = S[i] * wc[i] - ac[i] * d + kc[i] * vc;
+      S[i + 1] = S[i + 1] * wc[i + 1] - ac[i + 1] * d + kc[i + 1] * vc;
+      S[i + 2] = S[i + 2] * wc[i + 2] - ac[i + 2] * d + kc[i + 2] * vc;
+      S[i + 3] = S[i + 3] * wc[i + 3] - ac[i + 3] * d + kc[i + 3] * vc;
+      e0 += S[i] * rc[i];
+      e1 += S[i + 1] * rc[i + 1];
+      e2 += S[i + 2] * rc[i + 2];
+      e3 += S[i + 3] * rc[i + 3];
+    }
+    const float od = quad_sum((e0 + e1) + (e2 + e3));
+    if (live && part == 0) o[((long)t * H + h) * Dv + col] = od;
+    if (PF) {
+#pragma unroll
+      for (int i = 0; i < KP; ++i) {
+        kc[i] = kx[i]; rc[i] = rx[i]; wc[i] = wx[i]; ac[i] = ax[i];
+      }
+      vc = vx;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < KP; ++i)
+      if (i0 + i < Dk) sp[(long)(i0 + i) * Dv + col] = S[i];
+  }
 }
 
 bool rows_ok(const torch::Tensor &t) {
@@ -522,10 +725,12 @@ bool rows_ok(const torch::Tensor &t) {
 
 void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                       torch::Tensor conv_state, torch::Tensor slots,
-                      torch::Tensor has_init, torch::Tensor query_start_loc) {
+                      torch::Tensor has_init, torch::Tensor query_start_loc,
+                      bool activation) {
   const long T = x.size(0);
   const int C = x.size(1);
   const int taps = w.size(1);
+  const int act = activation ? 1 : 0;
   const int B = slots.numel();
   if (T == 0) return;
   const auto st = x.scalar_type();
@@ -556,7 +761,7 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                      (const TT *)w.data_ptr(),                               \
                      (const TT *)conv_state.data_ptr(),                      \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
-                     query_start_loc.data_ptr<int>(), B, C)
+                     query_start_loc.data_ptr<int>(), B, C, act)
 #define CONV8_T(TT)                                                          \
   switch (taps) {                                                            \
     case 1: CONV8(TT, 1); break;                                             \
@@ -578,7 +783,7 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                        (const TT *)w.data_ptr(),                             \
                        (const TT *)conv_state.data_ptr(),                    \
                        slots.data_ptr<long>(), has_init.data_ptr<int>(),     \
-                       query_start_loc.data_ptr<int>(), B, C, taps);         \
+                       query_start_loc.data_ptr<int>(), B, C, taps, act);    \
   if (taps > 1)                                                              \
     hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3(B, cy),          \
                        dim3(256), 0, stream, (TT *)conv_state.data_ptr(),    \
@@ -691,13 +896,21 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
 }
 
 void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
-              torch::Tensor w, long H, double eps) {
-  const int Dv = w.numel();
+              torch::Tensor w, long H, double eps, bool sigmoid_gate,
+              double scale) {
+  TORCH_CHECK(o.dim() == 3 && o.size(1) == H, "rms_gate: o [T, H, Dv]");
+  const int Dv = o.size(2);
   const long rows = o.numel() / std::max(Dv, 1);
   if (rows == 0) return;
   const auto st = out.scalar_type();
   TORCH_CHECK(o.scalar_type() == at::kFloat && o.is_contiguous());
-  TORCH_CHECK(out.is_contiguous() && out.numel() == o.numel());
+  TORCH_CHECK(rows_ok(out) && out.size(0) * H == rows &&
+              out.size(1) == H * Dv, "rms_gate: out [T, H * Dv] rows");
+  TORCH_CHECK(w.numel() == Dv || w.numel() == H * Dv,
+              "rms_gate: weight [Dv] or [H * Dv]");
+  const int w_hs = w.numel() == Dv ? 0 : Dv;
+  const int sig = sigmoid_gate ? 1 : 0;
+  const long os = out.stride(0);
   TORCH_CHECK(rows_ok(z) && z.scalar_type() == st && z.size(1) == H * Dv &&
               z.size(0) * H == rows);
   TORCH_CHECK(w.scalar_type() == st && w.is_contiguous());
@@ -709,14 +922,16 @@ void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
       reinterpret_cast<uintptr_t>(z.data_ptr()) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(o.data_ptr()) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0 &&
+      (os * out.element_size()) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(w.data_ptr()) % 16 == 0;
   if (vec8) {
     const long blocks = (rows * lpr + 255) / 256;
 #define G8(TT, L)                                                            \
   hipLaunchKernelGGL((rms_gate8_kernel<TT, L>), dim3(blocks), dim3(256), 0,  \
-                     stream, (TT *)out.data_ptr(), o.data_ptr<float>(),      \
+                     stream, (TT *)out.data_ptr(), os, o.data_ptr<float>(),  \
                      (const TT *)z.data_ptr(), (long)z.stride(0),            \
-                     (const TT *)w.data_ptr(), (int)H, rows, (float)eps)
+                     (const TT *)w.data_ptr(), w_hs, (int)H, rows,           \
+                     (float)eps, sig, (float)scale)
 #define G8_L(TT)                                                             \
   switch (lpr) {                                                             \
     case 1: G8(TT, 1); break;                                                \
@@ -737,12 +952,142 @@ void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
   }
 #define RUN(TT)                                                              \
   hipLaunchKernelGGL((rms_gate_kernel<TT>), dim3(rows), dim3(64), 0, stream, \
-                     (TT *)out.data_ptr(), o.data_ptr<float>(),              \
+                     (TT *)out.data_ptr(), os, o.data_ptr<float>(),          \
                      (const TT *)z.data_ptr(), (long)z.stride(0),            \
-                     (const TT *)w.data_ptr(), (int)H, Dv, (float)eps)
+                     (const TT *)w.data_ptr(), w_hs, (int)H, Dv, (float)eps, \
+                     sig, (float)scale)
   if (st == at::kBFloat16) RUN(__hip_bfloat16);
   else if (st == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "rms_gate: bf16 or fp32");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+void token_shift(torch::Tensor out, torch::Tensor h, torch::Tensor mu,
+                 torch::Tensor state, torch::Tensor slots,
+                 torch::Tensor has_init, torch::Tensor query_start_loc,
+                 long max_query_len) {
+  const long T = h.size(0);
+  if (T == 0) return;
+  const int W = h.size(1);
+  const auto st = h.scalar_type();
+  const int B = slots.numel();
+  TORCH_CHECK(h.is_cuda() && rows_ok(h) && out.is_contiguous() &&
+              out.scalar_type() == st && out.numel() == T * W);
+  TORCH_CHECK(mu.is_contiguous() && mu.numel() == W && mu.scalar_type() == st);
+  TORCH_CHECK(state.is_contiguous() && state.dim() == 2 &&
+              state.size(1) == W && state.scalar_type() == st,
+              "token_shift: state [slots, width] in the dtype of h");
+  TORCH_CHECK(slots.scalar_type() == at::kLong && slots.is_contiguous());
+  TORCH_CHECK(has_init.scalar_type() == at::kInt && has_init.numel() == B);
+  TORCH_CHECK(query_start_loc.scalar_type() == at::kInt &&
+              query_start_loc.numel() >= B + 1);
+  auto stream = at::cuda::getCurrentCUDAStream();
+  const size_t es = h.element_size();
+  const bool vec8 =
+      W % 8 == 0 && (h.stride(0) * es) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(h.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(mu.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(state.data_ptr()) % 16 == 0;
+  // one token per sequence: the launch that shifts also rolls the state
+  const int store = (max_query_len == 1 && T == B) ? 1 : 0;
+  const int cy = vec8 ? (W / 8 + 255) / 256 : (W + 255) / 256;
+#define RUN(TT, E)                                                           \
+  hipLaunchKernelGGL((token_shift_kernel<TT, E>), dim3(T, cy), dim3(256), 0, \
+                     stream, (TT *)out.data_ptr(), (const TT *)h.data_ptr(), \
+                     (long)h.stride(0), (const TT *)mu.data_ptr(),           \
+                     (TT *)state.data_ptr(), slots.data_ptr<long>(),         \
+                     has_init.data_ptr<int>(),                               \
+                     query_start_loc.data_ptr<int>(), B, W, store)
+#define RUN_ALL(TT)                                                          \
+  if (vec8) RUN(TT, 8); else RUN(TT, 1);                                     \
+  if (!store)                                                                \
+    hipLaunchKernelGGL((shift_state_kernel<TT>), dim3(B, (W + 255) / 256),   \
+                       dim3(256), 0, stream, (TT *)state.data_ptr(),         \
+                       (const TT *)h.data_ptr(), (long)h.stride(0),          \
+                       slots.data_ptr<long>(),                               \
+                       query_start_loc.data_ptr<int>(), W)
+  if (st == at::kBFloat16) { RUN_ALL(__hip_bfloat16); }
+  else if (st == at::kFloat) { RUN_ALL(float); }
+  else TORCH_CHECK(false, "token_shift: bf16 or fp32");
+#undef RUN_ALL
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+void general_delta_rule(torch::Tensor o, torch::Tensor r, torch::Tensor k,
+                        torch::Tensor v, torch::Tensor w_logit,
+                        torch::Tensor a_logit, torch::Tensor w0,
+                        double decay_scale, torch::Tensor state,
+                        torch::Tensor slots, torch::Tensor has_init,
+                        torch::Tensor query_start_loc, long max_query_len) {
+  const long T = r.size(0);
+  if (T == 0) return;
+  const auto st = r.scalar_type();
+  TORCH_CHECK(state.dim() == 4 && state.scalar_type() == at::kFloat &&
+              state.is_contiguous());
+  const int H = state.size(1), Dk = state.size(2), Dv = state.size(3);
+  TORCH_CHECK(r.is_cuda() && rows_ok(r) && rows_ok(k) && rows_ok(v) &&
+              rows_ok(w_logit) && rows_ok(a_logit));
+  TORCH_CHECK(k.scalar_type() == st && v.scalar_type() == st &&
+              w_logit.scalar_type() == st && a_logit.scalar_type() == st &&
+              w0.scalar_type() == st);
+  TORCH_CHECK(r.size(1) == (long)H * Dk && k.size(1) == (long)H * Dk &&
+              v.size(1) == (long)H * Dv && w_logit.size(1) == (long)H * Dk &&
+              a_logit.size(1) == (long)H * Dk && w0.numel() == (long)H * Dk &&
+              w0.is_contiguous(), "general_delta_rule: operand widths");
+  TORCH_CHECK(k.size(0) == T && v.size(0) == T && w_logit.size(0) == T &&
+              a_logit.size(0) == T);
+  TORCH_CHECK(r.stride(0) == k.stride(0) && r.stride(0) == v.stride(0),
+              "r, k, v must share a row stride (slices of one buffer)");
+  TORCH_CHECK(o.scalar_type() == at::kFloat && o.is_contiguous() &&
+              o.numel() == T * H * Dv);
+  const int B = slots.numel();
+  TORCH_CHECK(slots.scalar_type() == at::kLong && slots.is_contiguous());
+  TORCH_CHECK(has_init.scalar_type() == at::kInt && has_init.numel() == B);
+  TORCH_CHECK(query_start_loc.scalar_type() == at::kInt &&
+              query_start_loc.numel() >= B + 1);
+  TORCH_CHECK(Dk <= 256, "general delta rule: key size <= 256");
+  auto stream = at::cuda::getCurrentCUDAStream();
+  auto prep = torch::empty({T, 2, H, Dk}, o.options().dtype(at::kFloat));
+#define PREP(TT)                                                             \
+  hipLaunchKernelGGL((general_delta_prep_kernel<TT>), dim3(T, H), dim3(64),  \
+                     0, stream, prep.data_ptr<float>(),                      \
+                     (const TT *)k.data_ptr(), (long)k.stride(0),            \
+                     (const TT *)w_logit.data_ptr(), (long)w_logit.stride(0), \
+                     (const TT *)a_logit.data_ptr(), (long)a_logit.stride(0), \
+                     (const TT *)w0.data_ptr(), H, Dk, (float)decay_scale)
+  if (st == at::kBFloat16) PREP(__hip_bfloat16);
+  else if (st == at::kFloat) PREP(float);
+  else TORCH_CHECK(false, "general_delta_rule: bf16 or fp32");
+#undef PREP
+  const dim3 grid(B, H, (Dv + 63) / 64);
+  const int kp = Dk <= 32 ? 8 : Dk <= 64 ? 16 : Dk <= 128 ? 32 : 64;
+  const size_t es = r.element_size();
+  // 16 B vector loads of the per-lane slices (operands and fp32 prep rows):
+  // every slice whole and every row / head / slice offset 16 B aligned
+  const int vec =
+      (Dk == 4 * kp && (r.stride(0) * es) % 16 == 0 && (Dk * es) % 16 == 0 &&
+       reinterpret_cast<uintptr_t>(r.data_ptr()) % 16 == 0 &&
+       reinterpret_cast<uintptr_t>(k.data_ptr()) % 16 == 0) ? 1 : 0;
+#define RUN(TT, KPV, PFV)                                                    \
+  hipLaunchKernelGGL((general_delta_kernel<TT, KPV, PFV>), grid, dim3(256),  \
+                     0, stream, o.data_ptr<float>(),                         \
+                     (const TT *)r.data_ptr(), (const TT *)k.data_ptr(),     \
+                     (const TT *)v.data_ptr(), (long)r.stride(0),            \
+                     prep.data_ptr<float>(), state.data_ptr<float>(),        \
+                     slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
+                     query_start_loc.data_ptr<int>(), H, Dk, Dv, vec)
+#define RUN_KP(TT)                                                           \
+  if (Dk <= 32) RUN(TT, 8, true);                                            \
+  else if (Dk <= 64) RUN(TT, 16, true);                                      \
+  else if (Dk <= 128) RUN(TT, 32, true);                                     \
+  else RUN(TT, 64, false)
+  if (st == at::kBFloat16) { RUN_KP(__hip_bfloat16); }
+  else if (st == at::kFloat) { RUN_KP(float); }
+  else TORCH_CHECK(false, "general_delta_rule: bf16 or fp32");
+#undef RUN_KP
 #undef RUN
   HIP_CHECK_KERNEL();
 }

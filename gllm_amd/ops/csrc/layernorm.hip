@@ -7,6 +7,9 @@
 //   layernorm_f32:      h = LN_pre(x)                       x fp32 -> h T
 //   residual_layernorm: x += LN_post(y); h = LN_pre(x)      y T, x fp32
 //                       with a gate: LN_post sees y * sigmoid(gate)
+//   stream_rmsnorm:     the RMS form (plain weight, eps inside the root,
+//                       no mean): x += mult * RMS(s (y + y2)) w_post;
+//                       x += add; h = RMS(x) w_pre — every part optional
 //
 // One workgroup per token row; the row lives in LDS as fp32 between the
 // mean, variance (mean of squared deviations, two passes: no E[x^2] -
@@ -383,6 +386,200 @@ void residual_layernorm(torch::Tensor x, torch::Tensor y,
   if (st == at::kBFloat16) RUN(__hip_bfloat16);
   else if (st == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "residual_layernorm: bf16 or fp32 sublayer output");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+namespace {
+
+// RMS sandwich boundary, one workgroup per token row, the row in LDS:
+//   z = y_scale * (y + y2);  x += mult * z / sqrt(mean z^2 + eps) * w_post
+//   x += add (one fp32 row for all tokens);  h = x / sqrt(mean x^2 + eps) * w_pre
+// y == nullptr skips the first line, h == nullptr the last.
+template <typename T>
+__global__ __launch_bounds__(LN_BLOCK) void stream_rmsnorm_kernel(
+    float *__restrict__ x, const T *__restrict__ y, long y_stride,
+    const T *__restrict__ y2, long y2_stride, const T *__restrict__ w_post,
+    const float *__restrict__ add, T *__restrict__ h,
+    const T *__restrict__ w_pre, float eps, float mult, float y_scale,
+    int width, int vec) {
+  extern __shared__ float row[];
+  __shared__ float red[LN_BLOCK / WAVE_SIZE];
+  const long base = (long)blockIdx.x * width;
+  const int tid = threadIdx.x;
+  float ss = 0.f;
+  if (y) {
+    const T *yr = y + (long)blockIdx.x * y_stride;
+    const T *y2r = y2 ? y2 + (long)blockIdx.x * y2_stride : nullptr;
+    if (vec) {
+      for (int i = tid * 8; i < width; i += LN_BLOCK * 8) {
+        float a[8], b[8];
+        ld8<T>(yr + i, a);
+        if (y2r) {
+          ld8<T>(y2r + i, b);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) a[e] += b[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          a[e] *= y_scale;
+          row[i + e] = a[e];
+          ss += a[e] * a[e];
+        }
+      }
+    } else {
+      for (int i = tid; i < width; i += LN_BLOCK) {
+        float a = ScalarOps<T>::to_f32(yr[i]);
+        if (y2r) a += ScalarOps<T>::to_f32(y2r[i]);
+        a *= y_scale;
+        row[i] = a;
+        ss += a * a;
+      }
+    }
+    const float inv = mult / sqrtf(ln_block_sum(ss, red) / width + eps);
+    ss = 0.f;
+    // each thread revisits exactly the elements it wrote above
+    if (vec) {
+      for (int i = tid * 8; i < width; i += LN_BLOCK * 8) {
+        float wf[8], xf[8], af[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        ld8<T>(w_post + i, wf);
+        ld8<float>(x + base + i, xf);
+        if (add) ld8<float>(add + i, af);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          xf[e] += row[i + e] * inv * wf[e];
+          xf[e] += af[e];
+          row[i + e] = xf[e];
+          ss += xf[e] * xf[e];
+        }
+        st8<float>(x + base + i, xf);
+      }
+    } else {
+      for (int i = tid; i < width; i += LN_BLOCK) {
+        float r = x[base + i] + row[i] * inv * ScalarOps<T>::to_f32(w_post[i]);
+        if (add) r += add[i];
+        x[base + i] = r;
+        row[i] = r;
+        ss += r * r;
+      }
+    }
+  } else {
+    if (vec) {
+      for (int i = tid * 8; i < width; i += LN_BLOCK * 8) {
+        float xf[8], af[8];
+        ld8<float>(x + base + i, xf);
+        if (add) {
+          ld8<float>(add + i, af);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) xf[e] += af[e];
+          st8<float>(x + base + i, xf);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          row[i + e] = xf[e];
+          ss += xf[e] * xf[e];
+        }
+      }
+    } else {
+      for (int i = tid; i < width; i += LN_BLOCK) {
+        float r = x[base + i];
+        if (add) {
+          r += add[i];
+          x[base + i] = r;
+        }
+        row[i] = r;
+        ss += r * r;
+      }
+    }
+  }
+  if (h == nullptr) return;
+  const float inv = 1.0f / sqrtf(ln_block_sum(ss, red) / width + eps);
+  if (vec) {
+    for (int i = tid * 8; i < width; i += LN_BLOCK * 8) {
+      float wf[8], of[8];
+      ld8<T>(w_pre + i, wf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) of[e] = row[i + e] * inv * wf[e];
+      st8<T>(h + base + i, of);
+    }
+  } else {
+    for (int i = tid; i < width; i += LN_BLOCK)
+      h[base + i] = ScalarOps<T>::from_f32(row[i] * inv *
+                                           ScalarOps<T>::to_f32(w_pre[i]));
+  }
+}
+
+}  // namespace
+
+void stream_rmsnorm(torch::Tensor x, c10::optional<torch::Tensor> y,
+                    c10::optional<torch::Tensor> y2,
+                    c10::optional<torch::Tensor> w_post,
+                    c10::optional<torch::Tensor> add,
+                    c10::optional<torch::Tensor> h,
+                    c10::optional<torch::Tensor> w_pre, double eps,
+                    double mult, double y_scale) {
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == at::kFloat &&
+              x.is_contiguous());
+  const int width = x.size(-1);
+  const long rows = x.numel() / std::max(width, 1);
+  if (rows == 0) return;
+  TORCH_CHECK(width > 0 && width * 4 <= 64 * 1024);
+  TORCH_CHECK(y.has_value() || h.has_value() || add.has_value());
+  at::ScalarType st = at::kFloat;
+  if (y.has_value()) st = y->scalar_type();
+  else if (h.has_value()) st = h->scalar_type();
+  const size_t es = st == at::kFloat ? 4 : 2;
+  const void *yp = nullptr, *y2p = nullptr, *wpost = nullptr, *wpre = nullptr;
+  const float *addp = nullptr;
+  void *hp = nullptr;
+  long ys = 0, y2s = 0;
+  bool vec = width % 8 == 0 && aligned16(x.data_ptr());
+  auto rows_of = [&](const torch::Tensor &t, const char *what) {
+    TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.size(0) == rows &&
+                t.size(1) == width && t.stride(1) == 1 &&
+                t.scalar_type() == st, "stream_rmsnorm: ", what,
+                " must be [rows, width] in the sublayer dtype");
+    vec = vec && aligned16(t.data_ptr()) && (t.stride(0) * es) % 16 == 0;
+  };
+  if (y.has_value()) {
+    rows_of(*y, "y");
+    TORCH_CHECK(w_post.has_value());
+    check_vec(*w_post, width, st);
+    yp = y->data_ptr(); ys = y->stride(0);
+    wpost = w_post->data_ptr();
+    vec = vec && aligned16(wpost);
+    if (y2.has_value()) {
+      rows_of(*y2, "y2");
+      y2p = y2->data_ptr(); y2s = y2->stride(0);
+    }
+  }
+  if (add.has_value()) {
+    TORCH_CHECK(add->is_cuda() && add->scalar_type() == at::kFloat &&
+                add->is_contiguous() && add->numel() == width,
+                "stream_rmsnorm: add must be fp32 [width]");
+    addp = add->data_ptr<float>();
+    vec = vec && aligned16(addp);
+  }
+  if (h.has_value()) {
+    TORCH_CHECK(w_pre.has_value());
+    TORCH_CHECK(h->is_contiguous() && h->numel() == x.numel() &&
+                h->scalar_type() == st);
+    check_vec(*w_pre, width, st);
+    hp = h->data_ptr();
+    wpre = w_pre->data_ptr();
+    vec = vec && aligned16(hp) && aligned16(wpre);
+  }
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(T)                                                              \
+  hipLaunchKernelGGL((stream_rmsnorm_kernel<T>), dim3(rows), dim3(LN_BLOCK), \
+                     width * sizeof(float), stream, x.data_ptr<float>(),    \
+                     (const T *)yp, ys, (const T *)y2p, y2s,                \
+                     (const T *)wpost, addp, (T *)hp, (const T *)wpre,      \
+                     (float)eps, (float)mult, (float)y_scale, width,        \
+                     vec ? 1 : 0)
+  if (st == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (st == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "stream_rmsnorm: bf16 or fp32");
 #undef RUN
   HIP_CHECK_KERNEL();
 }

@@ -408,6 +408,148 @@ __global__ __launch_bounds__(256) void topk_softmax_rows_kernel(
   }
 }
 
+// Sigmoid router with a selection-only correction and group limits.
+// One wave per token, up to 64 * TK_MAXJ experts, lane l holds experts
+// l, l + 64, ...: s = sigmoid(logit) weighs, c = s + correction chooses.
+// Experts form n_group equal groups of neighbours; a group scores the
+// sum of its two largest c and only experts of the `keep` best groups
+// stay eligible (the rest count as -inf). k rounds of a wave-wide
+// arg-max (ties to the lower index) pick the experts; weights are the
+// chosen s over their sum (+ 1e-20), times scale.
+// The per-wave LDS row holds c for the group scan.
+__global__ __launch_bounds__(256) void sigmoid_group_topk_kernel(
+    float *__restrict__ weights, int *__restrict__ ids,
+    const float *__restrict__ logits, const float *__restrict__ correction,
+    long rows, int E, int k, int n_group, int keep, float scale) {
+  extern __shared__ float sg_lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const long r = (long)blockIdx.x * 4 + wave;
+  if (r >= rows) return;  // no block-wide barrier below
+  float *crow = sg_lds + (size_t)wave * (E + n_group);
+  float *gsc = crow + E;
+  const float *row = logits + r * E;
+  float s[TK_MAXJ], c[TK_MAXJ];
+#pragma unroll
+  for (int j = 0; j < TK_MAXJ; ++j) {
+    const int e = lane + 64 * j;
+    if (e < E) {
+      s[j] = 1.0f / (1.0f + expf(-row[e]));
+      c[j] = s[j] + (correction ? correction[e] : 0.f);
+      crow[e] = c[j];
+    } else {
+      s[j] = 0.f;
+      c[j] = -INFINITY;
+    }
+  }
+  if (n_group > 1) {
+    const int per = E / n_group;
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // LDS writes of this wave landed
+    for (int g = lane; g < n_group; g += 64) {
+      float b0 = -INFINITY, b1 = -INFINITY;
+      for (int i = 0; i < per; ++i) {
+        const float x = crow[g * per + i];
+        if (x > b0) { b1 = b0; b0 = x; }
+        else if (x > b1) b1 = x;
+      }
+      gsc[g] = per > 1 ? b0 + b1 : b0;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+#pragma unroll
+    for (int j = 0; j < TK_MAXJ; ++j) {
+      const int e = lane + 64 * j;
+      if (e < E) {
+        const int g = e / per;
+        const float mine = gsc[g];
+        int rank = 0;  // groups ahead of mine; ties go to the lower index
+        for (int o = 0; o < n_group; ++o) {
+          const float x = gsc[o];
+          rank += (x > mine || (x == mine && o < g)) ? 1 : 0;
+        }
+        if (rank >= keep) c[j] = -INFINITY;
+      }
+    }
+  }
+  unsigned taken = 0;
+  float my_w = 0.f;
+  int my_idx = 0;
+  for (int it = 0; it < k; ++it) {
+    float best = -INFINITY, bs = 0.f;
+    int bidx = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < TK_MAXJ; ++j) {
+      const int e = lane + 64 * j;
+      if (e < E && !(taken >> j & 1u) && (bidx == 0x7fffffff || c[j] > best)) {
+        best = c[j];
+        bs = s[j];
+        bidx = e;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(best, off, 64);
+      const float os = __shfl_xor(bs, off, 64);
+      const int oi = __shfl_xor(bidx, off, 64);
+      const bool take = oi != 0x7fffffff &&
+                        (bidx == 0x7fffffff || ov > best ||
+                         (ov == best && oi < bidx) ||
+                         (best != best && ov == ov));
+      if (take) { best = ov; bs = os; bidx = oi; }
+    }
+    if ((bidx & 63) == lane) taken |= 1u << (bidx >> 6);
+    if (lane == it) { my_w = bs; my_idx = bidx; }
+  }
+  const float sum = wave_reduce_sum(lane < k ? my_w : 0.f);
+  if (lane < k) {
+    weights[r * k + lane] = my_w / (sum + 1e-20f) * scale;
+    ids[r * k + lane] = my_idx;
+  }
+}
+
+}  // namespace
+
+void sigmoid_group_topk(torch::Tensor weights, torch::Tensor ids,
+                        torch::Tensor logits,
+                        c10::optional<torch::Tensor> correction,
+                        long n_group, long keep, double scale) {
+  TORCH_CHECK(logits.is_cuda() && logits.dim() == 2 &&
+              logits.is_contiguous() && logits.scalar_type() == at::kFloat,
+              "logits: fp32 [rows, experts]");
+  const long rows = logits.size(0);
+  const int E = logits.size(1);
+  TORCH_CHECK(weights.dim() == 2 && weights.size(0) == rows &&
+              weights.is_contiguous() && weights.scalar_type() == at::kFloat);
+  const int k = weights.size(1);
+  TORCH_CHECK(ids.is_contiguous() && ids.scalar_type() == at::kInt &&
+              ids.numel() == rows * k);
+  TORCH_CHECK(E >= 1 && E <= 64 * TK_MAXJ && k >= 1 && k <= 64 && k <= E,
+              "sigmoid_group_topk: experts <= ", 64 * TK_MAXJ,
+              ", top <= min(64, experts)");
+  TORCH_CHECK(n_group >= 1 && E % n_group == 0 && keep >= 1 &&
+              keep <= n_group, "sigmoid_group_topk: bad groups");
+  TORCH_CHECK(k <= keep * (E / n_group),
+              "sigmoid_group_topk: the kept groups hold fewer experts "
+              "than are chosen");
+  const float *cp = nullptr;
+  if (correction.has_value()) {
+    TORCH_CHECK(correction->is_cuda() && correction->is_contiguous() &&
+                correction->scalar_type() == at::kFloat &&
+                correction->numel() == E, "correction: fp32 [experts]");
+    cp = correction->data_ptr<float>();
+  }
+  if (rows == 0) return;
+  auto stream = at::cuda::getCurrentCUDAStream();
+  const size_t lds = 4 * (size_t)(E + n_group) * sizeof(float);
+  hipLaunchKernelGGL(sigmoid_group_topk_kernel, dim3((rows + 3) / 4),
+                     dim3(256), lds, stream, weights.data_ptr<float>(),
+                     ids.data_ptr<int>(), logits.data_ptr<float>(), cp, rows,
+                     E, k, (int)n_group, (int)keep, (float)scale);
+  HIP_CHECK_KERNEL();
+}
+
+namespace {
+
 }  // namespace
 
 void topk_softmax_rows(torch::Tensor weights, torch::Tensor ids,

@@ -366,7 +366,8 @@ def sigmoid_group_topk(logits, correction, topk, n_group, keep, scale):
 def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
                        mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
                        half_layout=False, norm_last=False, do_norm=True,
-                       v_freqs=None, norm_span=False, v_unit=False):
+                       v_freqs=None, norm_span=False, v_unit=False,
+                       q_out=None):
     """Per-head RMS norm (plain weight, or none when the weight is None)
     + rotary on q (in place) and k; k, v land in the paged cache rows
     ``slot_mapping``. ``k`` None: a layer that reads another layer's
@@ -409,7 +410,8 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
             return norm(rotate(xf), w)
         return rotate(norm(xf, w))
 
-    q.copy_(prep(q, q_w, H).reshape(T, H * D).to(q.dtype))
+    (q if q_out is None else q_out).copy_(
+        prep(q, q_w, H).reshape(T, H * D).to(q.dtype))
     if k is None:
         return
     rows = slot_mapping[:T]
