@@ -308,6 +308,35 @@ def gopetar_config(sz, vocab=32000, window=4096, streams=2):
             "vocab": vocab, "vocab_size": vocab, "width": sz["width"]}
 
 
+def sofunex_config(sz, vocab=32000, window=4096):
+    """Looped stack of parallel layers: 6 layers, the first two run
+    twice (8 layer runs). Left: convolved (4 taps) windowed attention
+    with the row-wide q/k norm, rotate-half rotary on half of each head
+    and unit values; right: the generalized delta rule at the delta
+    geometry of the size table (rank-64 decay branch). Group-limited
+    sigmoid MoE with a shared expert in every layer."""
+    H, G, D = sz["attn"]
+    dh, _, dk, _ = sz["delta"]
+    mlp = {"kind": "moe", "expert": {"ff": sz["ff"]},
+           "router": {"experts": sz["experts"], "top": sz["top"],
+                      "groups": {"count": 4, "keep": 2}, "scale": 2.0},
+           "shared": {"ff": sz["ff"]}}
+    layer = {"type": "parallel", "mlp": mlp, "mixer": {
+        "left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D,
+                 "scale": D ** -0.5, "conv": 4, "mask": {"size": window},
+                 "rot": {"dims": D // 2, "base": 1000000.0,
+                         "scaling": {"factor": 8.0}}},
+        "left_scale": 0.7,
+        "right": {"heads": dh, "dim": dk, "decay_rank": 64},
+        "right_scale": 1.2}}
+    n = sz["layers"] - 2
+    return {"architecture": "Sofunex", "embedding": {"scale": 1.0},
+            "layers": [layer] * n,
+            "loop": {"start": 0, "stop": 2, "times": 2},
+            "norm": {"eps": 1e-5}, "residual_mult": 0.5, "vocab": vocab,
+            "vocab_size": vocab, "width": sz["width"]}
+
+
 COMPARE_PAIRS = {
     "sudevik": (("sudevik", sudevik_config),
                 ("hybrid-gdn", hybrid_gdn_config)),
@@ -316,6 +345,13 @@ COMPARE_PAIRS = {
     # closest existing family: Sudevik (windowed sink attention beside a
     # recurrent mixer over the state pool, fp32 stream, routed experts)
     "gopetar": (("gopetar", gopetar_config),
+                ("sudevik", sudevik_config)),
+    # closest existing families: Gopetar (a windowed-attention branch
+    # beside a recurrent branch in every layer, MoE with a shared
+    # expert) and Sudevik (delta rule over the state pool, sandwich
+    # norms over an fp32 stream)
+    "sofunex": (("sofunex", sofunex_config),
+                ("gopetar", gopetar_config),
                 ("sudevik", sudevik_config)),
 }
 
@@ -330,6 +366,8 @@ MODELS["gukirax-w2048"] = ("Gukirax-w2048-8runs",
                            gukirax_config(COMPARE_SIZES["w2048"]))
 MODELS["gopetar-w2048"] = ("Gopetar-w2048-8L",
                            gopetar_config(COMPARE_SIZES["w2048"]))
+MODELS["sofunex-w2048"] = ("Sofunex-w2048-8runs",
+                           sofunex_config(COMPARE_SIZES["w2048"]))
 MODELS["sudevik-attn-w2048"] = (
     "Sudevik-attn-w2048-8L",
     sudevik_attention_config(COMPARE_SIZES["w2048"]))
@@ -469,7 +507,10 @@ def main():
                          "talking-heads attention) vs an attention-only "
                          "Sudevik stack of as many layer runs; 'gopetar' "
                          "= Gopetar (two streams, attention beside a "
-                         "minGRU, latent attention) vs Sudevik")
+                         "minGRU, latent attention) vs Sudevik; 'sofunex' "
+                         "= Sofunex (looped; convolved windowed attention "
+                         "beside a generalized delta rule) vs Gopetar and "
+                         "Sudevik")
     ap.add_argument("--compare-sizes", type=str, default="w2048,w1024")
     ap.add_argument("--compare-decode", type=str, default="1,32,128")
     ap.add_argument("--compare-prefill-batch", type=int, default=4)

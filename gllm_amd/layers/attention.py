@@ -183,11 +183,14 @@ class WindowAttention(nn.Module):
                 q_out=q_out)
         if q_out is not None:
             q = q_out
+        direct = out if (vrot is None and out_scale == 1.0) else None
         o = ops.window_attention(
             q, gate, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
             fctx.query_start_loc, self.scale, self.window,
             self.keep_first, self.sink, fctx.max_query_len,
-            sinks=self.sinks, softcap=self.softcap)
+            sinks=self.sinks, softcap=self.softcap, out=direct)
+        if direct is not None:
+            return out
         if vrot is not None:
             # turn every head's sum back by the query's own position
             return ops.rotate_scale_rows(

@@ -166,7 +166,8 @@ class ConvAttentionDeltaMixer(nn.Module):
             slots, init = state_rows(fctx, T, h.device)
             qkv = ops.causal_conv_silu(
                 qkv, self.conv_weight, fctx.ssm_pool.conv_state[ssm_id],
-                slots, init, fctx.query_start_loc, activation=False)
+                slots, init, fctx.query_start_loc, activation=False,
+                max_query_len=fctx.max_query_len)
         q, k, v = qkv.split(self.attn_sizes, dim=-1)
         R, c0 = self.R, self.conv_dim
         r, k2, v2, g, a = (proj[:, c0 + i * R:c0 + (i + 1) * R]

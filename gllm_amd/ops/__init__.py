@@ -968,13 +968,14 @@ def clamp_swiglu(x: torch.Tensor, limit: float,
 def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
                      query_start_loc, scale, window=0, keep_first=0,
                      sink=False, max_query_len=0, sinks=None,
-                     softcap=0.0) -> torch.Tensor:
+                     softcap=0.0, out=None) -> torch.Tensor:
     """Ragged paged attention over K [pages, page, G, D] / V [.., Dv]:
     sliding window with kept first tokens, optional softmax sink (+1 in
     the denominator; ``sinks`` fp32 [H]: exp(sinks[h]) instead), tanh
     score cap (``softcap`` > 0: cap * tanh(s / cap)) and fused sigmoid
     output gate. K and V may be the same tensor (attention over a
-    cached latent). Returns [T, H*Dv].
+    cached latent). Returns [T, H*Dv]; ``out`` may be a column block
+    of a wider buffer.
 
     Batches that hold prompt portions (``max_query_len`` > 1) in bf16
     with D == Dv in {64, 128} run the MFMA tile kernel shared with
@@ -986,7 +987,8 @@ def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
         T = q.shape[0]
         D, Dv = k_cache.shape[3], v_cache.shape[3]
         H = q.shape[1] // D
-        out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+        if out is None:
+            out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
         if (max_query_len > 1 and q.dtype == torch.bfloat16 and D == Dv
                 and D in (64, 128)):
             _seq_kernels().window_attention_mfma(
@@ -1006,10 +1008,14 @@ def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
             query_start_loc, scale, window, keep_first, sink, sinks,
             softcap)
         return out
-    return torch_ref.window_attention(q, gate, k_cache, v_cache,
-                                      block_table, seq_lens,
-                                      query_start_loc, scale, window,
-                                      keep_first, sink, sinks, softcap)
+    res = torch_ref.window_attention(q, gate, k_cache, v_cache,
+                                     block_table, seq_lens,
+                                     query_start_loc, scale, window,
+                                     keep_first, sink, sinks, softcap)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
 
 
 # --------------------------------------------------------------- talking heads
@@ -1062,15 +1068,17 @@ def relu2(x: torch.Tensor) -> torch.Tensor:
 
 # --------------------------------------------------------------- delta rule
 def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc,
-                     activation=True):
+                     activation=True, max_query_len=0):
     """Ragged short causal conv + silu (``activation`` False: the plain
     convolution); rolls ``conv_state`` rows ``slots`` in place. x may be
-    a column slice of a merged projection."""
+    a column slice of a merged projection. ``max_query_len`` == 1
+    (decode-only batch): the state is rolled by the same launch."""
     if x.is_cuda:
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
         _seq_kernels().causal_conv_silu(out, x, w, conv_state, slots,
                                         has_init, query_start_loc,
-                                        bool(activation))
+                                        bool(activation),
+                                        int(max_query_len))
         return out
     from gllm_amd.ops import gdn_ref
     return gdn_ref.causal_conv_silu(x, w, conv_state, slots, has_init,

@@ -481,7 +481,8 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_mfma_kernel(
 // Merge split partials: out[b,h,:] = sum_s w_s * partial[s,b,h,:]
 template <int D>
 __global__ void decode_merge_kernel(
-    __hip_bfloat16 *__restrict__ out,       // [B, Hq, D]
+    __hip_bfloat16 *__restrict__ out,       // [B, Hq, D] (row stride)
+    long out_stride,
     const float *__restrict__ partial_out,  // [S, B, Hq, D]
     const float *__restrict__ partial_lse,  // [S, B, Hq]
     int num_splits, int Hq, int sink,
@@ -511,7 +512,7 @@ __global__ void decode_merge_kernel(
         __bfloat162float(gate[(long)b * gate_stride + (long)h * D + d]);
     res *= 1.f / (1.f + __expf(-z));
   }
-  out[((long)b * Hq + h) * D + d] = __float2bfloat16(res);
+  out[(long)b * out_stride + (long)h * D + d] = __float2bfloat16(res);
 }
 
 template <int D, int G>
@@ -573,6 +574,7 @@ void launch_decode(torch::Tensor &out, const torch::Tensor &q,
   HIP_CHECK_KERNEL();
   hipLaunchKernelGGL((decode_merge_kernel<D>), dim3(B, Hq), dim3(D), 0,
                      stream, (__hip_bfloat16 *)out.data_ptr(),
+                     out.dim() == 2 ? (long)out.stride(0) : (long)Hq * D,
                      partial.data_ptr<float>(), lse.data_ptr<float>(), zdim,
                      Hq, sink ? 1 : 0, (const __hip_bfloat16 *)gate,
                      gate_stride, sinks);
@@ -634,9 +636,10 @@ bool window_attention_decode(torch::Tensor out, torch::Tensor q,
       q.dim() != 2 || q.size(1) % (D * Hkv) != 0)
     return false;
   const int G = q.size(1) / D / Hkv;
-  TORCH_CHECK(q.stride(1) == 1 && out.is_contiguous() &&
-              out.scalar_type() == at::kBFloat16 &&
-              out.numel() == (long)B * Hkv * G * D);
+  TORCH_CHECK(q.stride(1) == 1 && out.dim() == 2 && out.stride(1) == 1 &&
+              out.size(0) == B && out.size(1) == (long)Hkv * G * D &&
+              out.scalar_type() == at::kBFloat16,
+              "out: bf16 [B, H*D] rows (a column block is fine)");
   TORCH_CHECK(k_cache.scalar_type() == at::kBFloat16 &&
               v_cache.scalar_type() == at::kBFloat16 &&
               k_cache.is_contiguous() && v_cache.is_contiguous());

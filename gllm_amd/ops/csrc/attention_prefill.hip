@@ -42,7 +42,8 @@ DEV_INLINE int kswz(int row, int byte_off) {
 
 template <int D>
 __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
-    __hip_bfloat16 *__restrict__ out,            // [T, Hq, D]
+    __hip_bfloat16 *__restrict__ out,            // [T, Hq, D] (row stride)
+    long out_stride,
     const __hip_bfloat16 *__restrict__ q,        // [T, Hq, D] (row stride)
     const __hip_bfloat16 *__restrict__ k_cache,  // [P, ps, Hkv, D]
     const __hip_bfloat16 *__restrict__ v_cache,
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
     const int qrow = tile * BQ + wave * 16 + lhi * 4 + r;
     if (qrow >= q_len) continue;
     const float inv_l = (l_run[r] > 0.f) ? 1.f / l_run[r] : 0.f;
-    __hip_bfloat16 *op = out + ((long)(q_start + qrow) * Hq + h) * D;
+    __hip_bfloat16 *op = out + (long)(q_start + qrow) * out_stride + (long)h * D;
     if (gate != nullptr) {
       const __hip_bfloat16 *gp =
           gate + (long)(q_start + qrow) * gate_stride + (long)h * D;
@@ -325,11 +326,13 @@ void launch_prefill(torch::Tensor &out, torch::Tensor &q, int Hq, int D,
   const int Hkv = k_cache.size(2);
   const int B = seq_lens.size(0);
   const int q_tiles = (int)((max_query_len + BQ - 1) / BQ);
+  // a 2-D out may be a column block of a wider buffer
+  const long out_stride = out.dim() == 2 ? out.stride(0) : (long)Hq * D;
   auto stream = at::cuda::getCurrentCUDAStream();
 #define RUN(DV)                                                              \
   hipLaunchKernelGGL((paged_prefill_kernel<DV>), dim3(q_tiles, B, Hq),       \
                      dim3(BLOCK), 0, stream,                                 \
-                     (__hip_bfloat16 *)out.data_ptr(),                       \
+                     (__hip_bfloat16 *)out.data_ptr(), out_stride,           \
                      (const __hip_bfloat16 *)q.data_ptr(),                   \
                      (const __hip_bfloat16 *)k_cache.data_ptr(),             \
                      (const __hip_bfloat16 *)v_cache.data_ptr(),             \
@@ -389,8 +392,10 @@ void window_attention_mfma(torch::Tensor out, torch::Tensor q,
   const int H = q.size(1) / D;
   TORCH_CHECK(H % k_cache.size(2) == 0);
   TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous());
-  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == at::kBFloat16 &&
-              out.numel() == T * H * D);
+  TORCH_CHECK(out.dim() == 2 && out.stride(1) == 1 && out.size(0) == T &&
+              out.size(1) == (long)H * D &&
+              out.scalar_type() == at::kBFloat16,
+              "out: bf16 [T, H*D] rows (a column block is fine)");
   TORCH_CHECK(block_table.scalar_type() == at::kInt &&
               block_table.stride(1) == 1 &&
               seq_lens.scalar_type() == at::kInt &&

@@ -116,9 +116,18 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
       const T *row = is_q ? q + (long)t * q_stride : k + (long)t * k_stride;
       n = (is_q ? H : G) * D;
       ss = 0.f;
-      for (int i = lane; i < n; i += QK_BLOCK) {
-        const float x = ScalarOps<T>::to_f32(row[i]);
-        ss += x * x;
+      if (n % 8 == 0 && reinterpret_cast<uintptr_t>(row) % 16 == 0) {
+        for (int i = lane * 8; i < n; i += QK_BLOCK * 8) {  // 16 B loads
+          float x[8];
+          ld8<T>(row + i, x);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ss += x[e] * x[e];
+        }
+      } else {
+        for (int i = lane; i < n; i += QK_BLOCK) {
+          const float x = ScalarOps<T>::to_f32(row[i]);
+          ss += x * x;
+        }
       }
     }
     ss = wave_reduce_sum(ss);
@@ -163,7 +172,8 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
 // (key part) x (value column).
 template <typename T, int CT>  // CT: column threads, pow2 >= min(Dv,256)
 __global__ __launch_bounds__(ATT_BLOCK) void window_attention_kernel(
-    T *__restrict__ out, const T *__restrict__ q, long q_stride,
+    T *__restrict__ out, long out_stride, const T *__restrict__ q,
+    long q_stride,
     const T *__restrict__ gate, long gate_stride,
     const T *__restrict__ k_cache, const T *__restrict__ v_cache,
     const int *__restrict__ block_table, int bt_stride,
@@ -295,7 +305,7 @@ __global__ __launch_bounds__(ATT_BLOCK) void window_attention_kernel(
             gate[(long)t * gate_stride + (long)h * Dv + d]);
         o *= 1.0f / (1.0f + expf(-z));
       }
-      out[((long)t * H + h) * Dv + d] = ScalarOps<T>::from_f32(o);
+      out[(long)t * out_stride + (long)h * Dv + d] = ScalarOps<T>::from_f32(o);
     }
   }
 }
@@ -430,8 +440,9 @@ void window_attention(torch::Tensor out, torch::Tensor q,
               k_cache.scalar_type() == st && v_cache.scalar_type() == st);
   TORCH_CHECK(v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == page &&
               v_cache.size(2) == G);
-  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == st &&
-              out.numel() == T * H * Dv);
+  TORCH_CHECK(rows_ok(out) && out.scalar_type() == st && out.size(0) == T &&
+              out.size(1) == (long)H * Dv,
+              "out: [T, H*Dv] rows (a column block is fine)");
   TORCH_CHECK(block_table.scalar_type() == at::kInt && block_table.dim() == 2 &&
               block_table.stride(1) == 1);
   TORCH_CHECK(seq_lens.scalar_type() == at::kInt && seq_lens.is_contiguous());
@@ -464,7 +475,8 @@ void window_attention(torch::Tensor out, torch::Tensor q,
 #define RUN(TT, CTV)                                                         \
   hipLaunchKernelGGL((window_attention_kernel<TT, CTV>), dim3(T, H),         \
                      dim3(ATT_BLOCK), lds, stream, (TT *)out.data_ptr(),     \
-                     (const TT *)q.data_ptr(), (long)q.stride(0),            \
+                     (long)out.stride(0), (const TT *)q.data_ptr(),          \
+                     (long)q.stride(0),                                      \
                      (const TT *)gp, gs, (const TT *)k_cache.data_ptr(),     \
                      (const TT *)v_cache.data_ptr(),                         \
                      block_table.data_ptr<int>(), (int)block_table.stride(0), \

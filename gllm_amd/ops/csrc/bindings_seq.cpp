@@ -81,7 +81,7 @@ bool window_attention_decode(torch::Tensor out, torch::Tensor q,
 void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                       torch::Tensor conv_state, torch::Tensor slots,
                       torch::Tensor has_init, torch::Tensor query_start_loc,
-                      bool activation);
+                      bool activation, long max_query_len);
 void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                        torch::Tensor v, torch::Tensor a, torch::Tensor b,
                        torch::Tensor A_log, torch::Tensor dt_bias,

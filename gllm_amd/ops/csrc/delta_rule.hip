@@ -58,25 +58,30 @@ DEV_INLINE float silu_f(float z) { return z / (1.0f + expf(-z)); }
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
     T *__restrict__ out, const T *__restrict__ x, long x_stride,
-    const T *__restrict__ w, const T *__restrict__ state,
+    const T *__restrict__ w, T *__restrict__ state,
     const long *__restrict__ slots, const int *__restrict__ has_init,
-    const int *__restrict__ qsl, int B, int C, int taps, int act) {
+    const int *__restrict__ qsl, int B, int C, int taps, int act,
+    int store) {
   const int t = blockIdx.x;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int b = find_seq(qsl, B, t);
   const int r = t - qsl[b];  // offset inside this portion
   const bool init = has_init[b] != 0;
-  const T *st = state + ((long)slots[b] * C + c) * (taps - 1);
+  T *st = state + ((long)slots[b] * C + c) * (taps - 1);
   float acc = 0.f;
   for (int tap = 0; tap < taps; ++tap) {
     const int rel = r - (taps - 1 - tap);
-    float xv;
+    T raw;
     if (rel >= 0)
-      xv = ScalarOps<T>::to_f32(x[(long)(qsl[b] + rel) * x_stride + c]);
+      raw = x[(long)(qsl[b] + rel) * x_stride + c];
     else
-      xv = init ? ScalarOps<T>::to_f32(st[taps - 1 + rel]) : 0.f;
-    acc += xv * ScalarOps<T>::to_f32(w[(long)c * taps + tap]);
+      raw = init ? st[taps - 1 + rel] : ScalarOps<T>::from_f32(0.f);
+    // store != 0: every portion is one token, so this thread alone reads
+    // and rolls its channel's history (slot i <- what tap i + 1 just read)
+    if (store && tap > 0) st[tap - 1] = raw;
+    acc += ScalarOps<T>::to_f32(raw) *
+           ScalarOps<T>::to_f32(w[(long)c * taps + tap]);
   }
   // the activation output feeds 16-bit consumers in bf16 serving
   out[(long)t * C + c] = ScalarOps<T>::from_f32(act ? silu_f(acc) : acc);
@@ -88,9 +93,9 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
 template <typename T, int TAPS>
 __global__ __launch_bounds__(256) void causal_conv_silu8_kernel(
     T *__restrict__ out, const T *__restrict__ x, long x_stride,
-    const T *__restrict__ w, const T *__restrict__ state,
+    const T *__restrict__ w, T *__restrict__ state,
     const long *__restrict__ slots, const int *__restrict__ has_init,
-    const int *__restrict__ qsl, int B, int C, int act) {
+    const int *__restrict__ qsl, int B, int C, int act, int store) {
   const int t = blockIdx.x;
   const int c0 = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (c0 >= C) return;
@@ -118,6 +123,15 @@ __global__ __launch_bounds__(256) void causal_conv_silu8_kernel(
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += xv[e] * wf[e * TAPS + tap];
+    if (store && tap > 0) {
+      // one-token portions: this thread alone reads and rolls its
+      // channels' history (slot tap - 1 <- what tap just read; the
+      // 16-bit values survive the trip through fp32 unchanged)
+      T *st = state + ((long)slots[b] * C + c0) * (TAPS - 1);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        st[e * (TAPS - 1) + tap - 1] = ScalarOps<T>::from_f32(xv[e]);
+    }
   }
   if (act) {
 #pragma unroll
@@ -717,6 +731,153 @@ __global__ __launch_bounds__(256) void general_delta_kernel(
   }
 }
 
+// Prompt-portion form of general_delta_kernel: the 4 waves of a workgroup
+// share k, r and the fp32 decay / removal rows of their head, so tiles of
+// TT tokens are staged once per workgroup into LDS as fp32 (double
+// buffered: the next tile's global loads are in flight while the current
+// one is computed) and every lane reads its key slice with 16 B LDS
+// loads. The arithmetic per token is exactly general_delta_kernel's.
+// grid (B, H, ceil(Dv / 64)), block 256.
+template <typename T, int KP>
+__global__ __launch_bounds__(256) void general_delta_tiled_kernel(
+    float *__restrict__ o, const T *__restrict__ r, const T *__restrict__ k,
+    const T *__restrict__ v, long rkv_stride, const float *__restrict__ prep,
+    float *__restrict__ state, const long *__restrict__ slots,
+    const int *__restrict__ has_init, const int *__restrict__ qsl, int H,
+    int Dk, int Dv) {
+  constexpr int TT = KP == 64 ? 4 : 8;     // tokens per tile
+  constexpr int KPP = KP + 4;              // padded slice: no bank clash
+  constexpr int DKP = 4 * KP;              // padded key size
+  constexpr int ROW = 4 * KPP;             // one operand row in LDS
+  constexpr int TOK_F = 4 * ROW + 64;      // k | r | w | ak | v columns
+  constexpr int PER = TT * 2 * DKP / 256;  // k/r (and w/ak) per thread, tile
+  constexpr int VPER = TT * 64 / 256;
+  __shared__ __attribute__((aligned(16))) float lds[2][TT * TOK_F];
+
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int vcol = wave * 16 + (lane >> 2);  // column inside the 64 block
+  const int col = blockIdx.z * 64 + vcol;
+  const int part = lane & 3;
+  const int i0 = part * KP;
+  const int start = qsl[b], end = qsl[b + 1];
+  if (start >= end) return;
+  const bool live = col < Dv;
+  const int colc = live ? col : Dv - 1;
+  const long PW = 2L * H * Dk;
+
+  float *sp = state + ((long)slots[b] * H + h) * Dk * Dv;
+  float S[KP];
+  const bool init = has_init[b] != 0;
+#pragma unroll
+  for (int i = 0; i < KP; ++i)
+    S[i] = (init && i0 + i < Dk) ? sp[(long)(i0 + i) * Dv + colc] : 0.f;
+
+  T stg[PER];
+  float stg_f[PER];
+  T stg_v[VPER];
+  auto stage_load = [&](int tile0) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = j * 256 + tid;
+      const int tt = idx / (2 * DKP);
+      const int w = (idx / DKP) & 1;
+      const int i = idx % DKP;
+      const long t = tile0 + tt;
+      const bool ok = i < Dk && t < end;
+      const T *src = w ? r : k;
+      stg[j] = ok ? src[t * rkv_stride + (long)h * Dk + i]
+                  : ScalarOps<T>::from_f32(0.f);
+      stg_f[j] = ok ? prep[t * PW + ((long)w * H + h) * Dk + i] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < VPER; ++j) {
+      const int idx = j * 256 + tid;
+      const int tt = idx / 64, c = blockIdx.z * 64 + idx % 64;
+      const long t = tile0 + tt;
+      stg_v[j] = (c < Dv && t < end)
+                     ? v[t * rkv_stride + (long)h * Dv + c]
+                     : ScalarOps<T>::from_f32(0.f);
+    }
+  };
+  auto stage_store = [&](float *buf) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = j * 256 + tid;
+      const int tt = idx / (2 * DKP);
+      const int w = (idx / DKP) & 1;
+      const int i = idx % DKP;
+      float *tok = buf + tt * TOK_F + (i / KP) * KPP + i % KP;
+      tok[w * ROW] = ScalarOps<T>::to_f32(stg[j]);   // k (w = 0) | r
+      tok[(2 + w) * ROW] = stg_f[j];                 // decay | removal
+    }
+#pragma unroll
+    for (int j = 0; j < VPER; ++j) {
+      const int idx = j * 256 + tid;
+      buf[(idx / 64) * TOK_F + 4 * ROW + idx % 64] =
+          ScalarOps<T>::to_f32(stg_v[j]);
+    }
+  };
+
+  stage_load(start);
+  stage_store(lds[0]);
+  __syncthreads();
+  int cur = 0;
+  for (int tile0 = start; tile0 < end; tile0 += TT) {
+    const bool more = tile0 + TT < end;
+    if (more) stage_load(tile0 + TT);
+    const int n = end - tile0 < TT ? end - tile0 : TT;
+    const float *buf = lds[cur];
+    for (int tt = 0; tt < n; ++tt) {
+      const float *tok = buf + tt * TOK_F + part * KPP;
+      const floatx4 *kp4 = reinterpret_cast<const floatx4 *>(tok);
+      const floatx4 *rp4 = reinterpret_cast<const floatx4 *>(tok + ROW);
+      const floatx4 *wp4 = reinterpret_cast<const floatx4 *>(tok + 2 * ROW);
+      const floatx4 *ap4 = reinterpret_cast<const floatx4 *>(tok + 3 * ROW);
+      const float vc = buf[tt * TOK_F + 4 * ROW + vcol];
+      float kc[KP];
+      float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+      for (int i = 0; i < KP; i += 4) {
+        const floatx4 kk = kp4[i / 4];
+        kc[i] = kk[0]; kc[i + 1] = kk[1]; kc[i + 2] = kk[2]; kc[i + 3] = kk[3];
+        d0 += S[i] * kk[0];
+        d1 += S[i + 1] * kk[1];
+        d2 += S[i + 2] * kk[2];
+        d3 += S[i + 3] * kk[3];
+      }
+      const float d = quad_sum((d0 + d1) + (d2 + d3));
+      float e0 = 0.f, e1 = 0.f, e2 = 0.f, e3 = 0.f;
+#pragma unroll
+      for (int i = 0; i < KP; i += 4) {
+        const floatx4 rr = rp4[i / 4];
+        const floatx4 ww = wp4[i / 4];
+        const floatx4 aa = ap4[i / 4];
+        S[i] = S[i] * ww[0] - aa[0] * d + kc[i] * vc;
+        S[i + 1] = S[i + 1] * ww[1] - aa[1] * d + kc[i + 1] * vc;
+        S[i + 2] = S[i + 2] * ww[2] - aa[2] * d + kc[i + 2] * vc;
+        S[i + 3] = S[i + 3] * ww[3] - aa[3] * d + kc[i + 3] * vc;
+        e0 += S[i] * rr[0];
+        e1 += S[i + 1] * rr[1];
+        e2 += S[i + 2] * rr[2];
+        e3 += S[i + 3] * rr[3];
+      }
+      const float od = quad_sum((e0 + e1) + (e2 + e3));
+      if (live && part == 0)
+        o[((long)(tile0 + tt) * H + h) * Dv + col] = od;
+    }
+    if (more) stage_store(lds[cur ^ 1]);
+    __syncthreads();
+    cur ^= 1;
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < KP; ++i)
+      if (i0 + i < Dk) sp[(long)(i0 + i) * Dv + col] = S[i];
+  }
+}
+
 bool rows_ok(const torch::Tensor &t) {
   return t.dim() == 2 && t.stride(1) == 1;
 }
@@ -726,11 +887,14 @@ bool rows_ok(const torch::Tensor &t) {
 void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                       torch::Tensor conv_state, torch::Tensor slots,
                       torch::Tensor has_init, torch::Tensor query_start_loc,
-                      bool activation) {
+                      bool activation, long max_query_len) {
   const long T = x.size(0);
   const int C = x.size(1);
   const int taps = w.size(1);
   const int act = activation ? 1 : 0;
+  // one token per sequence: the convolution's launch also rolls the state
+  const int store = (max_query_len == 1 && T == slots.numel() &&
+                     w.size(1) > 1) ? 1 : 0;
   const int B = slots.numel();
   if (T == 0) return;
   const auto st = x.scalar_type();
@@ -758,10 +922,9 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   hipLaunchKernelGGL((causal_conv_silu8_kernel<TT, TP>), dim3(T, cy8),       \
                      dim3(256), 0, stream, (TT *)out.data_ptr(),             \
                      (const TT *)x.data_ptr(), (long)x.stride(0),            \
-                     (const TT *)w.data_ptr(),                               \
-                     (const TT *)conv_state.data_ptr(),                      \
+                     (const TT *)w.data_ptr(), (TT *)conv_state.data_ptr(),  \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
-                     query_start_loc.data_ptr<int>(), B, C, act)
+                     query_start_loc.data_ptr<int>(), B, C, act, store)
 #define CONV8_T(TT)                                                          \
   switch (taps) {                                                            \
     case 1: CONV8(TT, 1); break;                                             \
@@ -780,11 +943,11 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
     hipLaunchKernelGGL((causal_conv_silu_kernel<TT>), dim3(T, cy),           \
                        dim3(256), 0, stream, (TT *)out.data_ptr(),           \
                        (const TT *)x.data_ptr(), (long)x.stride(0),          \
-                       (const TT *)w.data_ptr(),                             \
-                       (const TT *)conv_state.data_ptr(),                    \
+                       (const TT *)w.data_ptr(), (TT *)conv_state.data_ptr(), \
                        slots.data_ptr<long>(), has_init.data_ptr<int>(),     \
-                       query_start_loc.data_ptr<int>(), B, C, taps, act);    \
-  if (taps > 1)                                                              \
+                       query_start_loc.data_ptr<int>(), B, C, taps, act,     \
+                       store);                                               \
+  if (taps > 1 && !store)                                                              \
     hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3(B, cy),          \
                        dim3(256), 0, stream, (TT *)conv_state.data_ptr(),    \
                        (const TT *)x.data_ptr(), (long)x.stride(0),          \
@@ -1079,8 +1242,24 @@ void general_delta_rule(torch::Tensor o, torch::Tensor r, torch::Tensor k,
                      prep.data_ptr<float>(), state.data_ptr<float>(),        \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
                      query_start_loc.data_ptr<int>(), H, Dk, Dv, vec)
+#define RUNT(TT, KPV)                                                        \
+  hipLaunchKernelGGL((general_delta_tiled_kernel<TT, KPV>), grid, dim3(256), \
+                     0, stream, o.data_ptr<float>(),                         \
+                     (const TT *)r.data_ptr(), (const TT *)k.data_ptr(),     \
+                     (const TT *)v.data_ptr(), (long)r.stride(0),            \
+                     prep.data_ptr<float>(), state.data_ptr<float>(),        \
+                     slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
+                     query_start_loc.data_ptr<int>(), H, Dk, Dv)
+  // batches that hold a prompt portion stage tiles through LDS; decode-
+  // only batches (one token per sequence) keep everything in registers
+  const bool tiled = max_query_len != 1;
 #define RUN_KP(TT)                                                           \
-  if (Dk <= 32) RUN(TT, 8, true);                                            \
+  if (tiled) {                                                               \
+    if (Dk <= 32) RUNT(TT, 8);                                               \
+    else if (Dk <= 64) RUNT(TT, 16);                                         \
+    else if (Dk <= 128) RUNT(TT, 32);                                        \
+    else RUNT(TT, 64);                                                       \
+  } else if (Dk <= 32) RUN(TT, 8, true);                                     \
   else if (Dk <= 64) RUN(TT, 16, true);                                      \
   else if (Dk <= 128) RUN(TT, 32, true);                                     \
   else RUN(TT, 64, false)
@@ -1088,6 +1267,7 @@ void general_delta_rule(torch::Tensor o, torch::Tensor r, torch::Tensor k,
   else if (st == at::kFloat) { RUN_KP(float); }
   else TORCH_CHECK(false, "general_delta_rule: bf16 or fp32");
 #undef RUN_KP
+#undef RUNT
 #undef RUN
   HIP_CHECK_KERNEL();
 }
