@@ -644,15 +644,18 @@ __global__ __launch_bounds__(64) void general_delta_prep_kernel(
 // lanes shares a column and splits the key axis in 4 slices of KP. Per token
 //   d = k^T S[:, col];  S[i, col] <- w_i S[i, col] - ak_i d + k_i v_col;
 //   o_col = r^T S[:, col]
-// PF: the next token's operands are loaded while this one is computed
-// (off for KP = 64, where they would not fit the register file).
-template <typename T, int KP, bool PF>
+// This is the form for decode-only batches (one token per sequence; it
+// walks longer portions too): no pre-pass, every lane forms decay and
+// removal rate of its own key slice from the logits, and the quad that
+// shares a column holds the whole key, so |k|^2 is one quad sum.
+template <typename T, int KP>
 __global__ __launch_bounds__(256) void general_delta_kernel(
     float *__restrict__ o, const T *__restrict__ r, const T *__restrict__ k,
-    const T *__restrict__ v, long rkv_stride, const float *__restrict__ prep,
-    float *__restrict__ state, const long *__restrict__ slots,
-    const int *__restrict__ has_init, const int *__restrict__ qsl, int H,
-    int Dk, int Dv, int vec) {
+    const T *__restrict__ v, long rkv_stride, const T *__restrict__ wl,
+    long wl_stride, const T *__restrict__ al, long al_stride,
+    const T *__restrict__ w0, float c, float *__restrict__ state,
+    const long *__restrict__ slots, const int *__restrict__ has_init,
+    const int *__restrict__ qsl, int H, int Dk, int Dv, int vec, int vec_l) {
   const int b = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = blockIdx.z * 64 + wave * 16 + (lane >> 2);
@@ -663,7 +666,6 @@ __global__ __launch_bounds__(256) void general_delta_kernel(
   const int colc = live ? col : Dv - 1;  // clamp loads, mask stores
   if (blockIdx.z * 64 + wave * 16 >= Dv) return;  // whole wave idle
   if (start >= end) return;
-  const long PW = 2L * H * Dk;
 
   float *sp = state + ((long)slots[b] * H + h) * Dk * Dv;
   float S[KP];
@@ -671,58 +673,44 @@ __global__ __launch_bounds__(256) void general_delta_kernel(
 #pragma unroll
   for (int i = 0; i < KP; ++i)
     S[i] = (init && i0 + i < Dk) ? sp[(long)(i0 + i) * Dv + colc] : 0.f;
+  float w0c[KP];
+  load_slice<T, KP>(w0 + (long)h * Dk, i0, Dk, vec_l, w0c);
 
-  float kc[KP], rc[KP], wc[KP], ac[KP];
-  float vc;
-  auto load_tok = [&](long t, float *kk, float *rr, float *ww, float *aa,
-                      float &vv) {
-    load_slice<T, KP>(k + t * rkv_stride + (long)h * Dk, i0, Dk, vec, kk);
-    load_slice<T, KP>(r + t * rkv_stride + (long)h * Dk, i0, Dk, vec, rr);
-    const float *pp = prep + t * PW + (long)h * Dk;
-    load_slice<float, KP>(pp, i0, Dk, vec, ww);
-    load_slice<float, KP>(pp + (long)H * Dk, i0, Dk, vec, aa);
-    vv = ScalarOps<T>::to_f32(v[t * rkv_stride + (long)h * Dv + colc]);
-  };
-  if (PF) load_tok(start, kc, rc, wc, ac, vc);
   for (int t = start; t < end; ++t) {
-    float kx[PF ? KP : 1], rx[PF ? KP : 1], wx[PF ? KP : 1], ax[PF ? KP : 1];
-    float vx = 0.f;
-    if (PF) {
-      // prefetch t + 1 (clamped: the last iteration re-reads row t)
-      load_tok(t + 1 < end ? t + 1 : t, kx, rx, wx, ax, vx);
-    } else {
-      load_tok(t, kc, rc, wc, ac, vc);
-    }
+    float kc[KP], rc[KP], wc[KP], ac[KP];
+    load_slice<T, KP>(k + t * rkv_stride + (long)h * Dk, i0, Dk, vec, kc);
+    load_slice<T, KP>(r + t * rkv_stride + (long)h * Dk, i0, Dk, vec, rc);
+    load_slice<T, KP>(wl + t * wl_stride + (long)h * Dk, i0, Dk, vec_l, wc);
+    load_slice<T, KP>(al + t * al_stride + (long)h * Dk, i0, Dk, vec_l, ac);
+    const float vc =
+        ScalarOps<T>::to_f32(v[t * rkv_stride + (long)h * Dv + colc]);
+    float ss = 0.f;
     float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;  // 4 chains, not one
 #pragma unroll
     for (int i = 0; i < KP; i += 4) {
+      ss += kc[i] * kc[i] + kc[i + 1] * kc[i + 1] + kc[i + 2] * kc[i + 2] +
+            kc[i + 3] * kc[i + 3];
       d0 += S[i] * kc[i];
       d1 += S[i + 1] * kc[i + 1];
       d2 += S[i + 2] * kc[i + 2];
       d3 += S[i + 3] * kc[i + 3];
     }
-    const float d = quad_sum((d0 + d1) + (d2 + d3));
-    float e0 = 0.f, e1 = 0.f, e2 = 0.f, e3 = 0.f;
+    const float ik2 = 1.0f / (quad_sum(ss) + 1e-6f);
+    const float d = quad_sum((d0 + d1) + (d2 + d3)) * ik2;
+    float e0 = 0.f, e1 = 0.f;
 #pragma unroll
-    for (int i = 0; i < KP; i += 4) {
-      S[i] = S[i] * wc[i] - ac[i] * d + kc[i] * vc;
-      S[i + 1] = S[i + 1] * wc[i + 1] - ac[i + 1] * d + kc[i + 1] * vc;
-      S[i + 2] = S[i + 2] * wc[i + 2] - ac[i + 2] * d + kc[i + 2] * vc;
-      S[i + 3] = S[i + 3] * wc[i + 3] - ac[i + 3] * d + kc[i + 3] * vc;
+    for (int i = 0; i < KP; i += 2) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const float w = expf(-c / (1.0f + expf(-(wc[i + u] + w0c[i + u]))));
+        const float a = 1.0f / (1.0f + expf(-ac[i + u]));
+        S[i + u] = S[i + u] * w - a * kc[i + u] * d + kc[i + u] * vc;
+      }
       e0 += S[i] * rc[i];
       e1 += S[i + 1] * rc[i + 1];
-      e2 += S[i + 2] * rc[i + 2];
-      e3 += S[i + 3] * rc[i + 3];
     }
-    const float od = quad_sum((e0 + e1) + (e2 + e3));
+    const float od = quad_sum(e0 + e1);
     if (live && part == 0) o[((long)t * H + h) * Dv + col] = od;
-    if (PF) {
-#pragma unroll
-      for (int i = 0; i < KP; ++i) {
-        kc[i] = kx[i]; rc[i] = rx[i]; wc[i] = wx[i]; ac[i] = ax[i];
-      }
-      vc = vx;
-    }
   }
   if (live) {
 #pragma unroll
@@ -1213,7 +1201,13 @@ void general_delta_rule(torch::Tensor o, torch::Tensor r, torch::Tensor k,
               query_start_loc.numel() >= B + 1);
   TORCH_CHECK(Dk <= 256, "general delta rule: key size <= 256");
   auto stream = at::cuda::getCurrentCUDAStream();
-  auto prep = torch::empty({T, 2, H, Dk}, o.options().dtype(at::kFloat));
+  // batches that hold a prompt portion stage tiles through LDS after a
+  // per-token pre-pass; decode-only batches (one token per sequence) keep
+  // everything in registers and form decay / removal rate in the lane
+  const bool tiled = max_query_len != 1;
+  torch::Tensor prep;
+  if (tiled) {
+    prep = torch::empty({T, 2, H, Dk}, o.options().dtype(at::kFloat));
 #define PREP(TT)                                                             \
   hipLaunchKernelGGL((general_delta_prep_kernel<TT>), dim3(T, H), dim3(64),  \
                      0, stream, prep.data_ptr<float>(),                      \
@@ -1221,27 +1215,37 @@ void general_delta_rule(torch::Tensor o, torch::Tensor r, torch::Tensor k,
                      (const TT *)w_logit.data_ptr(), (long)w_logit.stride(0), \
                      (const TT *)a_logit.data_ptr(), (long)a_logit.stride(0), \
                      (const TT *)w0.data_ptr(), H, Dk, (float)decay_scale)
-  if (st == at::kBFloat16) PREP(__hip_bfloat16);
-  else if (st == at::kFloat) PREP(float);
-  else TORCH_CHECK(false, "general_delta_rule: bf16 or fp32");
+    if (st == at::kBFloat16) PREP(__hip_bfloat16);
+    else if (st == at::kFloat) PREP(float);
+    else TORCH_CHECK(false, "general_delta_rule: bf16 or fp32");
 #undef PREP
+  }
   const dim3 grid(B, H, (Dv + 63) / 64);
   const int kp = Dk <= 32 ? 8 : Dk <= 64 ? 16 : Dk <= 128 ? 32 : 64;
   const size_t es = r.element_size();
-  // 16 B vector loads of the per-lane slices (operands and fp32 prep rows):
-  // every slice whole and every row / head / slice offset 16 B aligned
-  const int vec =
-      (Dk == 4 * kp && (r.stride(0) * es) % 16 == 0 && (Dk * es) % 16 == 0 &&
-       reinterpret_cast<uintptr_t>(r.data_ptr()) % 16 == 0 &&
-       reinterpret_cast<uintptr_t>(k.data_ptr()) % 16 == 0) ? 1 : 0;
-#define RUN(TT, KPV, PFV)                                                    \
-  hipLaunchKernelGGL((general_delta_kernel<TT, KPV, PFV>), grid, dim3(256),  \
-                     0, stream, o.data_ptr<float>(),                         \
-                     (const TT *)r.data_ptr(), (const TT *)k.data_ptr(),     \
-                     (const TT *)v.data_ptr(), (long)r.stride(0),            \
-                     prep.data_ptr<float>(), state.data_ptr<float>(),        \
+  // 16 B vector loads of the per-lane slices: every slice whole and every
+  // row / head / slice offset 16 B aligned (vec: r, k; vec_l: the logit
+  // rows and w0)
+  auto al16 = [](const torch::Tensor &t) {
+    return reinterpret_cast<uintptr_t>(t.data_ptr()) % 16 == 0;
+  };
+  const bool whole = Dk == 4 * kp && (Dk * es) % 16 == 0;
+  const int vec = (whole && (r.stride(0) * es) % 16 == 0 && al16(r) &&
+                   al16(k)) ? 1 : 0;
+  const int vec_l = (whole && (w_logit.stride(0) * es) % 16 == 0 &&
+                     (a_logit.stride(0) * es) % 16 == 0 && al16(w_logit) &&
+                     al16(a_logit) && al16(w0)) ? 1 : 0;
+#define RUN(TT, KPV)                                                         \
+  hipLaunchKernelGGL((general_delta_kernel<TT, KPV>), grid, dim3(256), 0,    \
+                     stream, o.data_ptr<float>(), (const TT *)r.data_ptr(),  \
+                     (const TT *)k.data_ptr(), (const TT *)v.data_ptr(),     \
+                     (long)r.stride(0), (const TT *)w_logit.data_ptr(),      \
+                     (long)w_logit.stride(0),                                \
+                     (const TT *)a_logit.data_ptr(),                         \
+                     (long)a_logit.stride(0), (const TT *)w0.data_ptr(),     \
+                     (float)decay_scale, state.data_ptr<float>(),            \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
-                     query_start_loc.data_ptr<int>(), H, Dk, Dv, vec)
+                     query_start_loc.data_ptr<int>(), H, Dk, Dv, vec, vec_l)
 #define RUNT(TT, KPV)                                                        \
   hipLaunchKernelGGL((general_delta_tiled_kernel<TT, KPV>), grid, dim3(256), \
                      0, stream, o.data_ptr<float>(),                         \
@@ -1250,19 +1254,16 @@ void general_delta_rule(torch::Tensor o, torch::Tensor r, torch::Tensor k,
                      prep.data_ptr<float>(), state.data_ptr<float>(),        \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
                      query_start_loc.data_ptr<int>(), H, Dk, Dv)
-  // batches that hold a prompt portion stage tiles through LDS; decode-
-  // only batches (one token per sequence) keep everything in registers
-  const bool tiled = max_query_len != 1;
 #define RUN_KP(TT)                                                           \
   if (tiled) {                                                               \
     if (Dk <= 32) RUNT(TT, 8);                                               \
     else if (Dk <= 64) RUNT(TT, 16);                                         \
     else if (Dk <= 128) RUNT(TT, 32);                                        \
     else RUNT(TT, 64);                                                       \
-  } else if (Dk <= 32) RUN(TT, 8, true);                                     \
-  else if (Dk <= 64) RUN(TT, 16, true);                                      \
-  else if (Dk <= 128) RUN(TT, 32, true);                                     \
-  else RUN(TT, 64, false)
+  } else if (Dk <= 32) RUN(TT, 8);                                           \
+  else if (Dk <= 64) RUN(TT, 16);                                            \
+  else if (Dk <= 128) RUN(TT, 32);                                           \
+  else RUN(TT, 64)
   if (st == at::kBFloat16) { RUN_KP(__hip_bfloat16); }
   else if (st == at::kFloat) { RUN_KP(float); }
   else TORCH_CHECK(false, "general_delta_rule: bf16 or fp32");
