@@ -16,7 +16,9 @@
 //                       v is turned by its own position over all of Dv);
 //                       span norm: ONE RMS over all heads of the token's
 //                       q (k) row with row-sized weights; unit values:
-//                       each value head divided by its RMS on the way in
+//                       each value head divided by its RMS on the way in.
+//                       The span form runs one workgroup per token
+//                       (qk_span_rope_store_kernel) while the rows fit LDS
 //   window_attention    ragged batch (prompt portions beside single
 //                       decode tokens) over the paged cache: position i
 //                       sees j <= i with i - j < window or j < keep_first;
@@ -162,6 +164,112 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
                 : k_cache + (slot_mapping[t] * G + (y - H)) * D;
   for (int i = lane; i < D; i += QK_BLOCK)
     dst[i] = ScalarOps<T>::from_f32(buf[i]);
+}
+
+// ------------------------------------------------------------------
+// Row-wide form: one workgroup per token prepares the whole q row, the
+// whole k row and all value heads. The token's cos / sin table is formed
+// once (fp64 angle) and shared by every head; a row is read once, summed
+// by the block for its one RMS, then normed (row-sized weights), turned
+// and written. LDS: [2 * half] table + [max(H, G) * D] row as fp32.
+// grid (tokens), block 256.
+constexpr int SPAN_BLOCK = 256;
+
+template <typename T>
+DEV_INLINE void span_row(float *row, const float *cs, const float *sn,
+                         float *red, const T *__restrict__ src,
+                         const T *__restrict__ w, T *__restrict__ dst,
+                         int heads, int D, int rot_dims, int half_layout,
+                         float eps, bool vec) {
+  const int n = heads * D, tid = threadIdx.x;
+  float ss = 0.f;
+  if (vec) {
+    for (int i = tid * 8; i < n; i += SPAN_BLOCK * 8) {
+      ld8<T>(src + i, row + i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += row[i + e] * row[i + e];
+    }
+  } else {
+    for (int i = tid; i < n; i += SPAN_BLOCK) {
+      const float x = ScalarOps<T>::to_f32(src[i]);
+      row[i] = x;
+      ss += x * x;
+    }
+  }
+  __syncthreads();  // red may still be read from the previous row
+  const float inv =
+      1.0f / sqrtf(block_reduce_sum<SPAN_BLOCK>(ss, red) / n + eps);
+  const int half = rot_dims / 2;
+  // the turned pairs of every head
+  for (int idx = tid; idx < heads * half; idx += SPAN_BLOCK) {
+    const int h = idx / half, p = idx % half;
+    const int ia = h * D + (half_layout ? p : 2 * p);
+    const int ib = h * D + (half_layout ? p + half : 2 * p + 1);
+    const float a = row[ia] * inv * (w ? ScalarOps<T>::to_f32(w[ia]) : 1.0f);
+    const float b = row[ib] * inv * (w ? ScalarOps<T>::to_f32(w[ib]) : 1.0f);
+    dst[ia] = ScalarOps<T>::from_f32(a * cs[p] - b * sn[p]);
+    dst[ib] = ScalarOps<T>::from_f32(b * cs[p] + a * sn[p]);
+  }
+  // the dims that pass unchanged
+  const int rest = D - rot_dims;
+  for (int idx = tid; idx < heads * rest; idx += SPAN_BLOCK) {
+    const int i = (idx / rest) * D + rot_dims + idx % rest;
+    dst[i] = ScalarOps<T>::from_f32(
+        row[i] * inv * (w ? ScalarOps<T>::to_f32(w[i]) : 1.0f));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(SPAN_BLOCK) void qk_span_rope_store_kernel(
+    const T *__restrict__ q, long q_stride, const T *__restrict__ k,
+    long k_stride, const T *__restrict__ v, long v_stride,
+    const T *__restrict__ q_w, const T *__restrict__ k_w,
+    const long *__restrict__ positions, const long *__restrict__ slot_mapping,
+    const double *__restrict__ freqs, float mag, int rot_dims,
+    T *__restrict__ k_cache, T *__restrict__ v_cache, int H, int G, int D,
+    int Dv, float eps, int half_layout, int v_unit, T *__restrict__ q_out,
+    long q_out_stride, int vec_q, int vec_k) {
+  extern __shared__ float span_lds[];
+  __shared__ float red[SPAN_BLOCK / WAVE_SIZE];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int half = rot_dims / 2;
+  float *cs = span_lds, *sn = span_lds + half;
+  float *row = span_lds + ((2 * half + 3) & ~3);
+  const double pos = (double)positions[t];
+  for (int p = tid; p < half; p += SPAN_BLOCK) {
+    double s, c;
+    sincos(pos * freqs[p], &s, &c);
+    cs[p] = (float)c * mag;
+    sn[p] = (float)s * mag;
+  }
+  // (span_row's first barrier publishes the table)
+  span_row<T>(row, cs, sn, red, q + (long)t * q_stride, q_w,
+              q_out + (long)t * q_out_stride, H, D, rot_dims, half_layout,
+              eps, vec_q != 0);
+  if (k == nullptr) return;
+  const long slot = slot_mapping[t];
+  __syncthreads();  // every thread is done with the q row
+  span_row<T>(row, cs, sn, red, k + (long)t * k_stride, k_w,
+              k_cache + slot * G * D, G, D, rot_dims, half_layout, eps,
+              vec_k != 0);
+  // values: a wave per head
+  const int lane = tid & 63, wave = tid >> 6;
+  for (int g = wave; g < G; g += SPAN_BLOCK / WAVE_SIZE) {
+    const T *src = v + (long)t * v_stride + (long)g * Dv;
+    T *dst = v_cache + (slot * G + g) * Dv;
+    if (!v_unit) {
+      for (int i = lane; i < Dv; i += 64) dst[i] = src[i];
+      continue;
+    }
+    float vs = 0.f;
+    for (int i = lane; i < Dv; i += 64) {
+      const float x = ScalarOps<T>::to_f32(src[i]);
+      vs += x * x;
+    }
+    const float vinv = 1.0f / sqrtf(wave_reduce_sum(vs) / Dv + eps);
+    for (int i = lane; i < Dv; i += 64)
+      dst[i] = ScalarOps<T>::from_f32(ScalarOps<T>::to_f32(src[i]) * vinv);
+  }
 }
 
 // ------------------------------------------------------------------
@@ -401,6 +509,39 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
   }
   const int gy = own ? H + 2 * G : H;
   auto stream = at::cuda::getCurrentCUDAStream();
+  const long span_floats =
+      ((rot_dims + 3) & ~3L) + std::max(H, own ? G : 0L) * D;
+  if (norm_span && !vfp && span_floats * 4 <= 60 * 1024 && T >= 512) {
+    // prompt-sized batches, one workgroup per token: one cos / sin table
+    // and one read of each row for all heads (a handful of decode tokens
+    // is served sooner by the workgroup-per-head form below, which
+    // spreads a token over H + 2G workgroups)
+    const size_t es = q.element_size();
+    auto vec_ok = [&](const void *p, long stride, long n, const void *w) {
+      return n % 8 == 0 && (stride * es) % 16 == 0 &&
+             reinterpret_cast<uintptr_t>(p) % 16 == 0 ? 1 : 0;
+    };
+    const int vq = vec_ok(q.data_ptr(), q.stride(0), H * D, qwp);
+    const int vk = own ? vec_ok(kp, ks, G * D, kwp) : 0;
+#define RUNS(TT)                                                             \
+  hipLaunchKernelGGL((qk_span_rope_store_kernel<TT>), dim3(T),               \
+                     dim3(SPAN_BLOCK), span_floats * sizeof(float), stream,  \
+                     (const TT *)q.data_ptr(), (long)q.stride(0),            \
+                     (const TT *)kp, ks, (const TT *)vp, vs,                 \
+                     (const TT *)qwp, (const TT *)kwp,                       \
+                     positions.data_ptr<long>(),                             \
+                     own ? slot_mapping.data_ptr<long>() : nullptr,          \
+                     freqs.data_ptr<double>(), (float)mag, (int)rot_dims,    \
+                     (TT *)kcp, (TT *)vcp, (int)H, (int)G, (int)D, (int)Dv,  \
+                     (float)eps, half_layout ? 1 : 0, v_unit ? 1 : 0,        \
+                     (TT *)qop, qos, vq, vk)
+    if (st == at::kBFloat16) RUNS(__hip_bfloat16);
+    else if (st == at::kFloat) RUNS(float);
+    else TORCH_CHECK(false, "qk_norm_rope_store: bf16 or fp32");
+#undef RUNS
+    HIP_CHECK_KERNEL();
+    return;
+  }
 #define RUN(TT)                                                              \
   hipLaunchKernelGGL((qk_norm_rope_store_kernel<TT>), dim3(T, gy),           \
                      dim3(QK_BLOCK), D * sizeof(float), stream,              \

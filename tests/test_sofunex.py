@@ -481,6 +481,41 @@ def test_long_decoding(device, dtype):
     check_against_oracle(cfg, w, got, {"a": toks}, TOL[dtype])
 
 
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_long_prompt_and_its_continuation(device, dtype):
+    """A 540-token prompt in one step (the kernels that prompt-sized
+    batches select), the same prompt as 515 tokens + a portion of 2 +
+    single tokens, and as two long portions: the ends of the prompt and
+    places around both cuts against the oracle."""
+    cfg = make_config(stack_for(dtype, [
+        parallel(heads=4, kv_heads=2, dim=16, vdim=8, window=70,
+                 rot_dims=8, rheads=2, rdim=16, mlp=dense_ff(24)),
+        parallel(heads=2, kv_heads=1, dim=64, vdim=64, window=300,
+                 rot_dims=32, conv=4, rheads=1, rdim=32,
+                 mlp=moe_ff(experts=4, top=2, groups=(2, 1)))]),
+        width=32, vocab=50, loop=(0, 1, 2))
+    w = make_weights(cfg, 17)
+    llm = engine(save_model(cfg, w), device, dtype, max_tokens=1200)
+    toks = tokens_for(cfg, 540, 18)
+
+    def steps(rid, sizes):
+        out, lo = [], 0
+        for n in sizes:
+            want = [k for k in range(n)
+                    if lo + k in (0, 1, 69, 70, 71, 299, 300, 301, 511, 512,
+                                  513, 514, 515, 516, 517, 530, 538, 539)]
+            out.append({"entries": [(rid, toks[lo:lo + n], want)]})
+            lo += n
+        assert lo == 540
+        out[-1]["end"] = [rid]
+        return out
+
+    got = run_steps(llm, steps("whole", [540])
+                    + steps("tail", [515, 2] + [1] * 23)
+                    + steps("halves", [513, 27]), cfg["vocab"])
+    check_against_oracle(cfg, w, got, {r: toks for r in got}, TOL[dtype])
+
+
 def _paged(k, v, perm, page, npages):
     L, G, D = k.shape
     kc = torch.zeros(npages, page, G, D)
@@ -808,17 +843,19 @@ def test_routing_op(device):
     assert (w.cpu().sum(-1) - 1.0).abs().max() < 1e-5
 
 
+@pytest.mark.parametrize("T", [11, 600], ids=["t11", "t600"])
 @pytest.mark.parametrize("device,dtype", DEVICES)
-def test_span_norm_and_unit_values(device, dtype):
+def test_span_norm_and_unit_values(device, dtype, T):
     """ops.qk_norm_rope_store with one RMS over the whole q (k) row,
     rotate-half on a prefix of the head and unit-RMS values, against
     the oracle's pieces, rows scattered over pages in a shuffled order.
     One head is scaled up a thousandfold: a per-head norm would hide
-    that, the row norm shrinks every other head."""
+    that, the row norm shrinks every other head. 600 rows reach the
+    workgroup-per-token kernel of prompt-sized batches."""
     from gllm_amd import ops
     tdt = getattr(torch, dtype)
     g = torch.Generator().manual_seed(13)
-    T, H, G, D, Dv, dims, eps = 11, 4, 2, 12, 10, 8, 1e-5
+    H, G, D, Dv, dims, eps = 4, 2, 12, 10, 8, 1e-5
     q = torch.randn(T, H * D, generator=g)
     q[:, :D] *= 1000.0
     k = torch.randn(T, G * D, generator=g)
@@ -827,11 +864,12 @@ def test_span_norm_and_unit_values(device, dtype):
     kw = 1 + 0.3 * torch.randn(G * D, generator=g)
     q, k, v, qw, kw = (x.to(tdt) for x in (q, k, v, qw, kw))
     pos = torch.arange(5, 5 + T)
-    slot = torch.randperm(64, generator=g)[:T]
+    npages = T // 16 + 4
+    slot = torch.randperm(npages * 16, generator=g)[:T]
     freqs = (50.0 ** (-2.0 * torch.arange(dims // 2, dtype=torch.float64)
                       / dims)) / 2.0
-    kc = torch.zeros(4, 16, G, D, dtype=tdt, device=device)
-    vc = torch.zeros(4, 16, G, Dv, dtype=tdt, device=device)
+    kc = torch.zeros(npages, 16, G, D, dtype=tdt, device=device)
+    vc = torch.zeros(npages, 16, G, Dv, dtype=tdt, device=device)
     q_out = torch.zeros(T, H * D, dtype=tdt, device=device)
     ops.qk_norm_rope_store(
         q.to(device), k.to(device), v.to(device), qw.to(device),
