@@ -87,8 +87,9 @@ class ConvAttentionDeltaMixer(nn.Module):
     def __init__(self, width: int, m, eps: float, dtype):
         super().__init__()
         left, right = _get(m, "left"), _get(m, "right")
-        H, G = int(_get(left, "heads")), int(_get(left, "kv_heads"))
-        D, Dv = int(_get(left, "dim")), int(_get(left, "vdim"))
+        H, D = int(_get(left, "heads")), int(_get(left, "dim"))
+        G = int(_get(left, "kv_heads", H) or H)
+        Dv = int(_get(left, "vdim", D) or D)
         Hr, Dr = int(_get(right, "heads")), int(_get(right, "dim"))
         self.R = R = Hr * Dr
         self.kv_shape = (G, D, Dv)
@@ -100,7 +101,10 @@ class ConvAttentionDeltaMixer(nn.Module):
         self.y_scale = self.left_scale if self.left_scale != 0.0 else 1.0
         self.left_mul = self.left_scale / self.y_scale
         self.right_mul = self.right_scale / self.y_scale
-        self.taps = int(_get(left, "conv", 1) or 1)
+        # taps of the short convolution; 0 = the layer has none (a
+        # one-tap convolution is a per-channel factor and keeps its
+        # weights)
+        self.taps = int(_get(left, "conv", 0) or 0)
         self.attn_sizes = [H * D, G * D, G * Dv]
         self.conv_dim = sum(self.attn_sizes)
         # the decay's low-rank width comes with the checkpoint; the
@@ -113,7 +117,7 @@ class ConvAttentionDeltaMixer(nn.Module):
         self._pending = []      # tensors that arrived before w1
         if self.rank:
             self._size(self.rank)
-        if self.taps > 1:
+        if self.taps >= 1:
             self.conv_weight = nn.Parameter(
                 torch.zeros(self.conv_dim, self.taps, dtype=dtype),
                 requires_grad=False)
@@ -130,7 +134,7 @@ class ConvAttentionDeltaMixer(nn.Module):
                                 _get(rot, "scaling"))
         mask = _get(left, "mask")
         self.attn = WindowAttention(
-            -1, H, G, D, Dv, float(_get(left, "scale")), eps,
+            -1, H, G, D, Dv, float(_get(left, "scale", D ** -0.5)), eps,
             window=int(_get(mask, "size", 0) or 0), sink=False,
             rotary=rotary, params_dtype=dtype, qk_norm=True,
             norm_span=True, value_unit_norm=True)
@@ -152,8 +156,8 @@ class ConvAttentionDeltaMixer(nn.Module):
             self.w2.to(dev)
 
     def spec(self, width: int) -> SSMLayerSpec:
-        return self.delta.spec(self.conv_dim if self.taps > 1 else 0,
-                               self.taps, shift_dim=width)
+        return self.delta.spec(self.conv_dim if self.taps >= 1 else 0,
+                               max(self.taps, 1), shift_dim=width)
 
     def forward(self, h: torch.Tensor, fctx: ForwardContext, kv_index: int,
                 ssm_id: int):
@@ -161,7 +165,7 @@ class ConvAttentionDeltaMixer(nn.Module):
         T = h.shape[0]
         proj = self.in_proj(h)
         qkv = proj[:, :self.conv_dim]
-        if self.taps > 1 and not fctx.is_profile_run \
+        if self.taps >= 1 and not fctx.is_profile_run \
                 and fctx.ssm_pool is not None:
             slots, init = state_rows(fctx, T, h.device)
             qkv = ops.causal_conv_silu(
@@ -489,7 +493,7 @@ class SofunexForCausalLM(nn.Module):
             return True
         if side == "left":
             if sub[1:] == ["conv"] and sub[0] in ("q", "k", "v") \
-                    and mix.taps > 1:
+                    and mix.taps >= 1:
                 off = sum(mix.attn_sizes[:shard])
                 self._copy(mix.conv_weight.data.narrow(0, off, w.shape[0]),
                            w)

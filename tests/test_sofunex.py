@@ -101,7 +101,7 @@ def make_weights(cfg, seed):
         for n, rows in (("q", H * D), ("k", G * D), ("v", G * Dv)):
             lin(p + "mix.left." + n, rows, W, 2.0 if n != "v" else 1.0)
             vec(p + "mix.left.%s.b" % n, rows)
-            if a.get("conv", 1) > 1:
+            if a.get("conv"):
                 w[p + "mix.left.%s.conv" % n] = torch.randn(
                     rows, a["conv"], generator=g) / a["conv"] ** 0.5
         vec(p + "mix.left.q.norm", H * D, 0.3, 1.0)
@@ -299,6 +299,7 @@ MECHANISMS = {
                   window=1, conv=None)], None),
     "rot0-nowindow-taps5": (
         [parallel(rot_dims=0, vdim=20, window=None, conv=5)], None),
+    "one-tap": ([parallel(conv=1, rdim=16)], None),
     "right-one-head-odd-dim": (
         [parallel(rheads=1, rdim=7, rank=1)], None),
     "right-dim40-scales-one": (
