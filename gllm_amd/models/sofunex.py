@@ -176,7 +176,7 @@ class ConvAttentionDeltaMixer(nn.Module):
         R, c0 = self.R, self.conv_dim
         r, k2, v2, g, a = (proj[:, c0 + i * R:c0 + (i + 1) * R]
                            for i in range(5))
-        w_logit = self.w2(torch.tanh(proj[:, c0 + 5 * R:]))
+        w_logit = self.w2(ops.tanh_rows(proj[:, c0 + 5 * R:]))
         both = torch.empty(T, self.heads_out + R, dtype=h.dtype,
                            device=h.device)
         self.attn(q, k, v, None, fctx, out=both[:, :self.heads_out],

@@ -826,6 +826,16 @@ def gated_act_mul(x: torch.Tensor, act: str = "silu") -> torch.Tensor:
     return torch_ref.gelu_tanh_and_mul(x)
 
 
+def tanh_rows(x: torch.Tensor) -> torch.Tensor:
+    """tanh of x [rows, n] (a column block of a wider buffer is fine),
+    contiguous result in x's dtype."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _seq_kernels().tanh_rows(out, x)
+        return out
+    return torch.tanh(x.float()).to(x.dtype)
+
+
 def sigmoid_group_topk(logits: torch.Tensor, correction, topk: int,
                        n_group: int = 1, keep: int = 1,
                        scale: float = 1.0):

@@ -109,6 +109,7 @@ void stream_rmsnorm(torch::Tensor x, c10::optional<torch::Tensor> y,
                     c10::optional<torch::Tensor> w_pre, double eps,
                     double mult, double y_scale);
 void gated_act_mul(torch::Tensor out, torch::Tensor x, long act);
+void tanh_rows(torch::Tensor out, torch::Tensor x);
 void sigmoid_group_topk(torch::Tensor weights, torch::Tensor ids,
                         torch::Tensor logits,
                         c10::optional<torch::Tensor> correction,
@@ -174,6 +175,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("stream_rmsnorm", &stream_rmsnorm,
         "x += mult * RMS(y) w_post (+ add); h = RMS(x) w_pre");
   m.def("gated_act_mul", &gated_act_mul, "act(x[:d]) * x[d:], silu or gelu");
+  m.def("tanh_rows", &tanh_rows, "tanh over strided rows");
   m.def("sigmoid_group_topk", &sigmoid_group_topk,
         "sigmoid router with correction and group limits");
   m.def("skinny_gemm", &skinny_gemm,

@@ -500,3 +500,44 @@ void gated_act_mul(torch::Tensor out, torch::Tensor x, long act) {
 #undef RUN
   HIP_CHECK_KERNEL();
 }
+
+namespace {
+
+// out[r, i] = tanh(x[r, i]) over strided rows (a column block of a merged
+// projection), any width; the function is taken in fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void tanh_rows_kernel(
+    T *__restrict__ out, const T *__restrict__ x, long x_stride, long rows,
+    int n) {
+  const long total = rows * n;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long r = idx / n;
+    const int i = idx % n;
+    out[idx] = ScalarOps<T>::from_f32(
+        tanhf(ScalarOps<T>::to_f32(x[r * x_stride + i])));
+  }
+}
+
+}  // namespace
+
+void tanh_rows(torch::Tensor out, torch::Tensor x) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.stride(1) == 1,
+              "tanh_rows: x [rows, n] rows");
+  const long rows = x.size(0);
+  const int n = x.size(1);
+  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == x.scalar_type() &&
+              out.numel() == rows * n);
+  if (rows == 0 || n == 0) return;
+  const int grid = (int)std::min<long>((rows * n + 255) / 256, 8192);
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT)                                                              \
+  hipLaunchKernelGGL((tanh_rows_kernel<TT>), dim3(grid), dim3(256), 0,       \
+                     stream, (TT *)out.data_ptr(), (const TT *)x.data_ptr(), \
+                     (long)x.stride(0), rows, n)
+  if (x.scalar_type() == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (x.scalar_type() == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "tanh_rows: bf16 or fp32");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
